@@ -1,0 +1,129 @@
+"""Build the native parts of flux_amd in-tree for gfx950.
+
+  libfluxmi_kernels.so   HIP kernels + C-ABI (include/fluxmi.h)       <- flux_amd/csrc/kernels/*.hip
+  flux_ths_pybind*.so    C++ torch extension with Flux's op surface    <- flux_amd/csrc/ths_op/*.cc
+
+Usage: python -m flux_amd.build [--kernels-only] [--force]
+Outputs land in flux_amd/lib/ and travel with the source tree; nothing is installed.
+"""
+import argparse
+import concurrent.futures
+import os
+import subprocess
+import sys
+import sysconfig
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+PKG = os.path.join(ROOT, "flux_amd")
+KERNEL_DIR = os.path.join(PKG, "csrc", "kernels")
+THS_DIR = os.path.join(PKG, "csrc", "ths_op")
+LIB_DIR = os.path.join(PKG, "lib")
+OBJ_DIR = os.path.join(PKG, "lib", "obj")
+INCLUDE = os.path.join(ROOT, "include")
+
+ARCH = "gfx950"
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+# -packed-fp32-ops is switched off on purpose: the compiler must not form v_pk_*_f32 by itself.
+HIP_FLAGS = [
+    f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", f"-I{INCLUDE}",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+KERNEL_LIB = os.path.join(LIB_DIR, "libfluxmi_kernels.so")
+
+
+def _run(cmd):
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in proc.stdout.splitlines() if "packed-fp32-ops" not in l)
+    if proc.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), out))
+    return out
+
+
+def _newer(target, sources):
+    if not os.path.exists(target):
+        return False
+    t = os.path.getmtime(target)
+    return all(os.path.getmtime(s) <= t for s in sources)
+
+
+def build_kernels(force=True):
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    srcs = sorted(f for f in os.listdir(KERNEL_DIR) if f.endswith(".hip"))
+    deps = [os.path.join(KERNEL_DIR, f) for f in os.listdir(KERNEL_DIR)] + [os.path.join(INCLUDE, "fluxmi.h")]
+    if not force and _newer(KERNEL_LIB, deps):
+        return KERNEL_LIB
+
+    def compile_one(name):
+        obj = os.path.join(OBJ_DIR, name[:-4] + ".o")
+        _run([HIPCC, *HIP_FLAGS, "-c", os.path.join(KERNEL_DIR, name), "-o", obj])
+        return obj
+
+    with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(srcs))) as pool:
+        objs = list(pool.map(compile_one, srcs))
+    _run([HIPCC, f"--offload-arch={ARCH}", "-shared", "-fPIC", *objs, "-o", KERNEL_LIB])
+    return KERNEL_LIB
+
+
+def ths_ext_path():
+    suffix = sysconfig.get_config_var("EXT_SUFFIX") or ".so"
+    return os.path.join(LIB_DIR, "flux_ths_pybind" + suffix)
+
+
+def build_ths_op(force=True):
+    """C++ host layer: Flux's torch-extension op surface over the C-ABI (no device code in it)."""
+    import torch
+    from torch.utils import cpp_extension
+
+    srcs = sorted(os.path.join(THS_DIR, f) for f in os.listdir(THS_DIR) if f.endswith(".cc"))
+    if not srcs:
+        return None
+    out = ths_ext_path()
+    deps = srcs + [os.path.join(THS_DIR, f) for f in os.listdir(THS_DIR) if f.endswith(".h")]
+    deps.append(os.path.join(INCLUDE, "fluxmi.h"))
+    if not force and _newer(out, deps):
+        return out
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    inc = [f"-I{p}" for p in cpp_extension.include_paths()]
+    inc += [f"-I{INCLUDE}", f"-I{sysconfig.get_paths()['include']}", "-I/opt/rocm/include"]
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    cxx11 = int(torch._C._GLIBCXX_USE_CXX11_ABI)
+    flags = [
+        "-O2", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+        f"-D_GLIBCXX_USE_CXX11_ABI={cxx11}", "-DTORCH_EXTENSION_NAME=flux_ths_pybind",
+        "-DTORCH_API_INCLUDE_EXTENSION_H", "-Wno-deprecated-declarations",
+    ]
+
+    def compile_one(src):
+        obj = os.path.join(OBJ_DIR, "ths_" + os.path.basename(src)[:-3] + ".o")
+        _run(["g++", *flags, *inc, "-c", src, "-o", obj])
+        return obj
+
+    with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(srcs))) as pool:
+        objs = list(pool.map(compile_one, srcs))
+    _run([
+        "g++", "-shared", *objs, "-o", out, f"-L{torch_lib}", f"-L{LIB_DIR}",
+        "-ltorch", "-ltorch_cpu", "-ltorch_hip", "-ltorch_python", "-lc10", "-lc10_hip", "-lfluxmi_kernels",
+        "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{torch_lib}",
+    ])
+    return out
+
+
+def build_all(force=True, kernels_only=False):
+    libs = [build_kernels(force)]
+    if not kernels_only:
+        ext = build_ths_op(force)
+        if ext:
+            libs.append(ext)
+    return libs
+
+
+if __name__ == "__main__":
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--kernels-only", action="store_true")
+    ap.add_argument("--no-force", action="store_true", help="skip targets newer than their sources")
+    a = ap.parse_args()
+    for lib in build_all(force=not a.no_force, kernels_only=a.kernels_only):
+        print("built", os.path.relpath(lib, ROOT))
+    sys.exit(0)

@@ -1,0 +1,199 @@
+"""ctypes binding of the C-ABI in include/fluxmi.h.
+
+Thin on purpose: arguments are torch tensors (device memory + the current HIP stream come from
+PyTorch-ROCm), every call goes straight to libfluxmi_kernels.so and a non-zero status becomes a
+RuntimeError carrying fluxmi_last_error().  There is no fallback: a missing library raises on load.
+"""
+import ctypes
+import os
+
+import torch
+
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libfluxmi_kernels.so")
+_lib = None
+
+BF16 = 0
+FP8_E4M3 = 1
+
+EXPORTS = (
+    "fluxmi_version", "fluxmi_last_error", "fluxmi_device_cu_count",
+    "fluxmi_moe_route_sort_workspace_bytes", "fluxmi_moe_route_sort", "fluxmi_moe_gather_index",
+    "fluxmi_grouped_gemm_workspace_bytes", "fluxmi_grouped_gemm",
+    "fluxmi_topk_gather_reduce", "fluxmi_quant_e4m3_rowwise",
+)
+
+
+class GroupedGemmArgs(ctypes.Structure):
+    _fields_ = [
+        ("dtype", ctypes.c_int32), ("nexperts", ctypes.c_int32), ("max_rows", ctypes.c_int32),
+        ("n", ctypes.c_int32), ("k", ctypes.c_int32), ("a_rows", ctypes.c_int32),
+        ("a", ctypes.c_void_p), ("b", ctypes.c_void_p), ("d", ctypes.c_void_p),
+        ("splits", ctypes.c_void_p), ("gather_a", ctypes.c_void_p), ("scatter_d", ctypes.c_void_p),
+        ("alpha", ctypes.c_void_p), ("row_scale", ctypes.c_void_p), ("col_scale", ctypes.c_void_p),
+        ("scalar_scale", ctypes.c_float), ("reserved1", ctypes.c_int32),
+        ("scalar_scale_dev", ctypes.c_void_p),
+    ]
+
+
+def lib_path():
+    return _LIB_PATH
+
+
+def load():
+    """Load libfluxmi_kernels.so (after torch, so that both share one HIP runtime)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_LIB_PATH):
+        raise RuntimeError(
+            f"{_LIB_PATH} is missing: build it with `python -m flux_amd.build` (there is no fallback path)")
+    lib = ctypes.CDLL(_LIB_PATH, mode=ctypes.RTLD_GLOBAL)
+    vp, i32, i64, f32, sz = ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64, ctypes.c_float, ctypes.c_size_t
+    lib.fluxmi_version.restype = ctypes.c_int
+    lib.fluxmi_last_error.restype = ctypes.c_char_p
+    lib.fluxmi_device_cu_count.restype = ctypes.c_int
+    lib.fluxmi_moe_route_sort_workspace_bytes.restype = sz
+    lib.fluxmi_moe_route_sort_workspace_bytes.argtypes = [i32, i32, i32]
+    lib.fluxmi_moe_route_sort.argtypes = [vp, i32, i32, i32, vp, vp, vp, vp, vp, vp, sz, vp]
+    lib.fluxmi_moe_gather_index.argtypes = [vp, i32, i32, vp, vp, vp]
+    lib.fluxmi_grouped_gemm_workspace_bytes.restype = sz
+    lib.fluxmi_grouped_gemm_workspace_bytes.argtypes = [ctypes.POINTER(GroupedGemmArgs)]
+    lib.fluxmi_grouped_gemm.argtypes = [ctypes.POINTER(GroupedGemmArgs), vp, sz, vp]
+    lib.fluxmi_topk_gather_reduce.argtypes = [ctypes.POINTER(vp), i32, vp, vp, f32, i32, i32, i32, vp, vp]
+    lib.fluxmi_quant_e4m3_rowwise.argtypes = [vp, i64, i64, i32, f32, vp, vp, i32, vp]
+    _lib = lib
+    return lib
+
+
+def _check(status, what):
+    if status != 0:
+        raise RuntimeError(f"{what} failed ({status}): {load().fluxmi_last_error().decode()}")
+
+
+def _ptr(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _dev_tensor(t, dtype, name):
+    if t is None:
+        return
+    if not t.is_cuda or not t.is_contiguous() or t.dtype != dtype:
+        raise ValueError(f"{name} must be a contiguous device tensor of {dtype}, got {t.dtype} on {t.device}")
+
+
+def route_sort(choosed, nexperts, want_gather=True, want_topk_index=True):
+    """-> (splits[E], offsets[E+1], scatter_index like choosed, gather_index[M], topk_index[M])."""
+    lib = load()
+    _dev_tensor(choosed, torch.int32, "choosed")
+    ntokens, topk = choosed.shape
+    dev = choosed.device
+    m = ntokens * topk
+    splits = torch.empty(nexperts, dtype=torch.int32, device=dev)
+    offsets = torch.empty(nexperts + 1, dtype=torch.int32, device=dev)
+    scatter = torch.empty_like(choosed)
+    gather = torch.empty(m, dtype=torch.int32, device=dev) if want_gather else None
+    tki = torch.empty(m, dtype=torch.int32, device=dev) if want_topk_index else None
+    ws_bytes = lib.fluxmi_moe_route_sort_workspace_bytes(ntokens, topk, nexperts)
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
+    _check(lib.fluxmi_moe_route_sort(_ptr(choosed), ntokens, topk, nexperts, _ptr(splits), _ptr(offsets),
+                                     _ptr(scatter), _ptr(gather), _ptr(tki), _ptr(ws), ws_bytes, _stream()),
+           "fluxmi_moe_route_sort")
+    return splits, offsets, scatter, gather, tki
+
+
+def gather_index(scatter_index, topk):
+    lib = load()
+    _dev_tensor(scatter_index, torch.int32, "scatter_index")
+    m = scatter_index.numel()
+    gather = torch.empty(m, dtype=torch.int32, device=scatter_index.device)
+    tki = torch.empty(m, dtype=torch.int32, device=scatter_index.device)
+    _check(lib.fluxmi_moe_gather_index(_ptr(scatter_index), m, topk, _ptr(gather), _ptr(tki), _stream()),
+           "fluxmi_moe_gather_index")
+    return gather, tki
+
+
+def grouped_gemm(a, b, splits, out=None, gather_a=None, scatter_d=None, alpha=None, row_scale=None,
+                 col_scale=None, scalar_scale=1.0, scalar_scale_dev=None, max_rows=None):
+    """D = grouped GEMM of A [rows_a, K] with B [E, N, K]; see fluxmi_grouped_gemm in include/fluxmi.h."""
+    lib = load()
+    if a.dtype == torch.bfloat16:
+        dtype = BF16
+    elif a.dtype == torch.float8_e4m3fn:
+        dtype = FP8_E4M3
+    else:
+        raise ValueError(f"unsupported input dtype {a.dtype}")
+    _dev_tensor(a, a.dtype, "a")
+    _dev_tensor(b, a.dtype, "b")
+    _dev_tensor(splits, torch.int32, "splits")
+    _dev_tensor(gather_a, torch.int32, "gather_a")
+    _dev_tensor(scatter_d, torch.int32, "scatter_d")
+    for nm, t in (("alpha", alpha), ("row_scale", row_scale), ("col_scale", col_scale),
+                  ("scalar_scale_dev", scalar_scale_dev)):
+        _dev_tensor(t, torch.float32, nm)
+    e, n, k = b.shape
+    if a.shape[1] != k:
+        raise ValueError(f"K mismatch: a {tuple(a.shape)} vs b {tuple(b.shape)}")
+    if max_rows is None:
+        max_rows = gather_a.numel() if gather_a is not None else a.shape[0]
+    if out is None:
+        out = torch.empty(max_rows, n, dtype=torch.bfloat16, device=a.device)
+    _dev_tensor(out, torch.bfloat16, "out")
+    if out.shape[0] < max_rows or out.shape[1] != n:
+        raise ValueError(f"out {tuple(out.shape)} too small for [{max_rows}, {n}]")
+    args = GroupedGemmArgs(
+        dtype=dtype, nexperts=e, max_rows=max_rows, n=n, k=k, a_rows=a.shape[0],
+        a=a.data_ptr(), b=b.data_ptr(), d=out.data_ptr(), splits=splits.data_ptr(),
+        gather_a=None if gather_a is None else gather_a.data_ptr(),
+        scatter_d=None if scatter_d is None else scatter_d.data_ptr(),
+        alpha=None if alpha is None else alpha.data_ptr(),
+        row_scale=None if row_scale is None else row_scale.data_ptr(),
+        col_scale=None if col_scale is None else col_scale.data_ptr(),
+        scalar_scale=float(scalar_scale), reserved1=0,
+        scalar_scale_dev=None if scalar_scale_dev is None else scalar_scale_dev.data_ptr())
+    _check(lib.fluxmi_grouped_gemm(ctypes.byref(args), None, 0, _stream()), "fluxmi_grouped_gemm")
+    return out
+
+
+def topk_gather_reduce(inputs, routing_idx, topk, row_weight=None, scale=1.0, out=None):
+    """out[t] = bf16(scale * sum_g sum_j w[r] * inputs[g][r]), r = routing_idx[t*topk+j]."""
+    lib = load()
+    if isinstance(inputs, torch.Tensor):
+        inputs = [inputs]
+    for g, t in enumerate(inputs):
+        _dev_tensor(t, torch.bfloat16, f"inputs[{g}]")
+    _dev_tensor(routing_idx, torch.int32, "routing_idx")
+    _dev_tensor(row_weight, torch.float32, "row_weight")
+    m, n = inputs[0].shape
+    if routing_idx.numel() % topk:
+        raise ValueError("routing_idx length is not a multiple of topk")
+    ntokens = routing_idx.numel() // topk
+    if out is None:
+        out = torch.empty(ntokens, n, dtype=torch.bfloat16, device=inputs[0].device)
+    ptrs = (ctypes.c_void_p * len(inputs))(*[t.data_ptr() for t in inputs])
+    _check(lib.fluxmi_topk_gather_reduce(ptrs, len(inputs), _ptr(routing_idx), _ptr(row_weight),
+                                         float(scale), ntokens, topk, n, _ptr(out), _stream()),
+           "fluxmi_topk_gather_reduce")
+    return out
+
+
+def quant_e4m3(x, block_cols=0, eps=0.0, permute_scale=False):
+    """-> (q fp8_e4m3fn like x, scale_inv fp32).  block_cols 0 = one scale per row, 128 = 1x128 blocks."""
+    lib = load()
+    _dev_tensor(x, torch.bfloat16, "x")
+    rows, cols = x.shape
+    q = torch.empty(rows, cols, dtype=torch.float8_e4m3fn, device=x.device)
+    if block_cols == 0:
+        si = torch.empty(rows, dtype=torch.float32, device=x.device)
+    else:
+        nb = (cols + block_cols - 1) // block_cols
+        if permute_scale:
+            si = torch.zeros((rows + 127) // 128, nb, 128, dtype=torch.float32, device=x.device)
+        else:
+            si = torch.empty(rows, nb, dtype=torch.float32, device=x.device)
+    _check(lib.fluxmi_quant_e4m3_rowwise(_ptr(x), rows, cols, block_cols, float(eps), _ptr(q), _ptr(si),
+                                         int(permute_scale), _stream()), "fluxmi_quant_e4m3_rowwise")
+    return q, si

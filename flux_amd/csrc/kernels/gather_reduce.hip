@@ -1,0 +1,160 @@
+// Top-k (weighted) gather-reduce: out[t,:] = bf16(scale * sum_g sum_j w[r_j] * in_g[r_j,:]).
+//
+// HBM-streaming kernel.  One workgroup owns one token row (or a column slab of it); every lane moves
+// 16-byte vectors (8 bf16), so a wave touches 1 KiB of contiguous row per instruction.  All top-k
+// source rows of a token are fetched before the first add so that topk*ngroups loads are in flight per
+// lane.  Source rows are read exactly once in the whole launch, hence the non-temporal loads.
+#include "common.hpp"
+
+namespace fluxmi {
+namespace {
+
+constexpr int kMaxGroups = 4;
+constexpr int kThreads = 256;
+
+struct GroupPtrs {
+  const uint16_t *p[kMaxGroups];
+};
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ void accumulate8(float (&acc)[8], const u32x4 v, const float w) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const uint32_t u = v[i];
+    acc[2 * i] = fmaf(w, __uint_as_float(u << 16), acc[2 * i]);
+    acc[2 * i + 1] = fmaf(w, __uint_as_float(u & 0xffff0000u), acc[2 * i + 1]);
+  }
+}
+
+// TOPK > 0: compile-time top-k (loads fully unrolled).  TOPK == 0: run-time top-k.
+template <int TOPK, int NGROUPS, bool WEIGHTED>
+__global__ __launch_bounds__(kThreads) void topk_gather_reduce_kernel(
+    GroupPtrs in, const int32_t *__restrict__ routing_idx, const float *__restrict__ row_weight,
+    float scale, int32_t topk_rt, int32_t nvec /* n / 8 */, uint16_t *__restrict__ out) {
+  const int t = blockIdx.x;
+  const int topk = TOPK > 0 ? TOPK : topk_rt;
+  const size_t row_vecs = static_cast<size_t>(nvec);
+
+  for (int v = blockIdx.y * kThreads + threadIdx.x; v < nvec; v += gridDim.y * kThreads) {
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if constexpr (TOPK > 0) {
+      u32x4 vals[NGROUPS][TOPK];
+      float w[TOPK];
+#pragma unroll
+      for (int j = 0; j < TOPK; ++j) {
+        const int32_t r = routing_idx[static_cast<size_t>(t) * TOPK + j];
+        w[j] = 0.f;
+        if (r >= 0) w[j] = WEIGHTED ? row_weight[r] : 1.f;
+#pragma unroll
+        for (int g = 0; g < NGROUPS; ++g) {
+          vals[g][j] = u32x4{0u, 0u, 0u, 0u};
+          if (r >= 0) {  // r is wave-uniform: a skipped (dropped) row costs no traffic
+            const u32x4 *src =
+                reinterpret_cast<const u32x4 *>(in.p[g]) + static_cast<size_t>(r) * row_vecs + v;
+            vals[g][j] = __builtin_nontemporal_load(src);
+          }
+        }
+      }
+#pragma unroll
+      for (int g = 0; g < NGROUPS; ++g) {
+#pragma unroll
+        for (int j = 0; j < TOPK; ++j) accumulate8(acc, vals[g][j], w[j]);
+      }
+    } else {
+      for (int g = 0; g < NGROUPS; ++g) {
+        for (int j = 0; j < topk; ++j) {
+          const int32_t r = routing_idx[static_cast<size_t>(t) * topk + j];
+          if (r < 0) continue;
+          const float w = WEIGHTED ? row_weight[r] : 1.f;
+          const u32x4 *src =
+              reinterpret_cast<const u32x4 *>(in.p[g]) + static_cast<size_t>(r) * row_vecs + v;
+          accumulate8(acc, __builtin_nontemporal_load(src), w);
+        }
+      }
+    }
+    u32x4 o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t lo = float_to_bf16_bits(acc[2 * i] * scale);
+      const uint32_t hi = float_to_bf16_bits(acc[2 * i + 1] * scale);
+      o[i] = lo | (hi << 16);
+    }
+    u32x4 *dst = reinterpret_cast<u32x4 *>(out) + static_cast<size_t>(t) * row_vecs + v;
+    __builtin_nontemporal_store(o, dst);
+  }
+}
+
+template <int TOPK, int NGROUPS>
+void launch(bool weighted, dim3 grid, hipStream_t s, const GroupPtrs &in, const int32_t *idx,
+            const float *w, float scale, int32_t topk, int32_t nvec, uint16_t *out) {
+  if (weighted)
+    hipLaunchKernelGGL((topk_gather_reduce_kernel<TOPK, NGROUPS, true>), grid, dim3(kThreads), 0, s,
+                       in, idx, w, scale, topk, nvec, out);
+  else
+    hipLaunchKernelGGL((topk_gather_reduce_kernel<TOPK, NGROUPS, false>), grid, dim3(kThreads), 0, s,
+                       in, idx, w, scale, topk, nvec, out);
+}
+
+template <int NGROUPS>
+void dispatch_topk(bool weighted, dim3 grid, hipStream_t s, const GroupPtrs &in, const int32_t *idx,
+                   const float *w, float scale, int32_t topk, int32_t nvec, uint16_t *out) {
+  switch (topk) {
+    case 1: launch<1, NGROUPS>(weighted, grid, s, in, idx, w, scale, topk, nvec, out); break;
+    case 2: launch<2, NGROUPS>(weighted, grid, s, in, idx, w, scale, topk, nvec, out); break;
+    case 4: launch<4, NGROUPS>(weighted, grid, s, in, idx, w, scale, topk, nvec, out); break;
+    case 6: launch<6, NGROUPS>(weighted, grid, s, in, idx, w, scale, topk, nvec, out); break;
+    case 8: launch<8, NGROUPS>(weighted, grid, s, in, idx, w, scale, topk, nvec, out); break;
+    default: launch<0, NGROUPS>(weighted, grid, s, in, idx, w, scale, topk, nvec, out); break;
+  }
+}
+
+}  // namespace
+}  // namespace fluxmi
+
+extern "C" int fluxmi_topk_gather_reduce(const void *const *in, int32_t ngroups,
+                                         const int32_t *routing_idx, const float *row_weight,
+                                         float scale, int32_t ntokens, int32_t topk, int32_t n,
+                                         void *out, void *stream) {
+  using namespace fluxmi;
+  FLUXMI_REQUIRE(in != nullptr && routing_idx != nullptr && out != nullptr, FLUXMI_ERR_INVALID_ARG,
+                 "topk_gather_reduce: null pointer argument");
+  FLUXMI_REQUIRE(ngroups >= 1 && ngroups <= kMaxGroups, FLUXMI_ERR_UNSUPPORTED,
+                 "topk_gather_reduce: ngroups=%d outside [1,%d]", ngroups, kMaxGroups);
+  FLUXMI_REQUIRE(topk >= 1 && topk <= 64, FLUXMI_ERR_UNSUPPORTED,
+                 "topk_gather_reduce: topk=%d outside [1,64]", topk);
+  FLUXMI_REQUIRE(ntokens >= 0 && n >= 0, FLUXMI_ERR_INVALID_ARG,
+                 "topk_gather_reduce: negative size (ntokens=%d, n=%d)", ntokens, n);
+  FLUXMI_REQUIRE(n % 8 == 0, FLUXMI_ERR_UNSUPPORTED, "topk_gather_reduce: n=%d is not a multiple of 8",
+                 n);
+  GroupPtrs gp{};
+  for (int g = 0; g < ngroups; ++g) {
+    FLUXMI_REQUIRE(in[g] != nullptr && aligned16(in[g]), FLUXMI_ERR_INVALID_ARG,
+                   "topk_gather_reduce: input group %d is null or not 16-byte aligned", g);
+    gp.p[g] = static_cast<const uint16_t *>(in[g]);
+  }
+  FLUXMI_REQUIRE(aligned16(out), FLUXMI_ERR_INVALID_ARG,
+                 "topk_gather_reduce: output is not 16-byte aligned");
+  if (ntokens == 0 || n == 0) return FLUXMI_OK;
+
+  const int32_t nvec = n / 8;
+  // One workgroup per token row; rows wider than 2 vectors per lane are split over blockIdx.y so
+  // that small token counts still fill the chip.
+  int ysplit = 1;
+  if (ntokens < 2048) {
+    ysplit = (nvec + kThreads - 1) / kThreads;
+    if (ysplit > 16) ysplit = 16;
+  }
+  const dim3 grid(static_cast<unsigned>(ntokens), static_cast<unsigned>(ysplit));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool weighted = row_weight != nullptr;
+  uint16_t *o = static_cast<uint16_t *>(out);
+  switch (ngroups) {
+    case 1: dispatch_topk<1>(weighted, grid, s, gp, routing_idx, row_weight, scale, topk, nvec, o); break;
+    case 2: dispatch_topk<2>(weighted, grid, s, gp, routing_idx, row_weight, scale, topk, nvec, o); break;
+    case 3: dispatch_topk<3>(weighted, grid, s, gp, routing_idx, row_weight, scale, topk, nvec, o); break;
+    default: dispatch_topk<4>(weighted, grid, s, gp, routing_idx, row_weight, scale, topk, nvec, o); break;
+  }
+  FLUXMI_HIP_CHECK(hipGetLastError());
+  return FLUXMI_OK;
+}

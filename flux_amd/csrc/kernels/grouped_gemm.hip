@@ -1,0 +1,469 @@
+// Grouped GEMM over ragged per-expert row counts: D[r,:] = scale(r,:) * A[gather(r),:] @ B[e(r)]^T.
+//
+// Persistent kernel, one 512-thread workgroup (8 waves, 2 per SIMD) per CU, macro tile 256 rows x 256
+// columns, k-step of 64 bytes per row (32 bf16 or 64 fp8).  Both operand tiles are staged in LDS by
+// direct-to-LDS global loads (no register staging) in a 4-deep ring; the row gather of A is folded into
+// the per-lane global address of those loads.  Each wave owns a 128x64 slice of the macro tile
+// (4x2 MFMA blocks of 32x32, fp32 accumulators).  The two waves that share a SIMD run one phase apart
+// ("ping-pong"): while one issues its LDS fragment reads and the next global loads, the other issues
+// MFMAs, and workgroup barriers keep them alternating.
+//
+// The MFMA "A" operand is the weight fragment and the "B" operand the activation fragment, i.e. the
+// hardware computes D^T blocks: a lane then holds, for one output row, four consecutive output columns
+// per accumulator quad, which makes the epilogue's stores 8-byte packed bf16x4.
+//
+// Tile schedule: every workgroup rebuilds the per-expert (row offset, tile offset) tables from the
+// device-resident `splits` in LDS, then walks logical tile ids assigned so that the workgroups of one
+// XCD (those with equal blockIdx % 8) take a run of consecutive tiles; tiles of an expert are ordered
+// column-major (all row tiles of one weight panel first), so an XCD's L2 sees a few weight panels
+// shared by all row tiles of the expert.
+#include "common.hpp"
+
+namespace fluxmi {
+namespace {
+
+constexpr int BM = 256;
+constexpr int BN = 256;
+constexpr int KBYTES = 64;                 // bytes of K per row per k-step
+constexpr int STAGES = 4;
+constexpr int DIST = STAGES - 1;           // prefetch distance in k-steps
+constexpr int TILE_BYTES = 256 * KBYTES;   // one operand tile of one stage: 16 KiB
+constexpr int STAGE_BYTES = 2 * TILE_BYTES;
+constexpr int NTHREADS = 512;
+constexpr int LOADS_PER_STAGE = 4;         // direct-to-LDS instructions per wave per stage
+constexpr int kMaxExperts = 1024;
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+struct GemmParams {
+  const uint8_t *a;
+  const uint8_t *b;
+  uint16_t *d;
+  const int32_t *splits;
+  const int32_t *gather_a;
+  const int32_t *scatter_d;
+  const float *alpha;
+  const float *row_scale;
+  const float *col_scale;
+  const float *scalar_dev;
+  float scalar;
+  int32_t nexperts;
+  int32_t max_rows;
+  int32_t a_rows;
+  int32_t n;
+  int32_t k;
+};
+
+#define FLUXMI_WAITCNT(vm, lgkm) \
+  __builtin_amdgcn_s_waitcnt(((vm)&15) | (((vm) >> 4) << 14) | (7 << 4) | ((lgkm) << 8))
+
+typedef __attribute__((address_space(3))) void *lds_ptr_t;
+typedef const __attribute__((address_space(1))) void *gbl_ptr_t;
+
+// One wave-wide direct-to-LDS load: lane l fetches 16 bytes from `src` (per lane) and the hardware
+// stores them at lds_base + 16*l (lds_base is wave-uniform).
+__device__ __forceinline__ void load_to_lds16(const uint8_t *src, uint8_t *lds_base) {
+  __builtin_amdgcn_global_load_lds((gbl_ptr_t)src, (lds_ptr_t)lds_base, 16, 0, 0);
+}
+
+// LDS tile layout: rows of 64 bytes, two rows per 128-byte line, the eight 16-byte slots of a line
+// xor-swizzled with the line number so that a 32-row column of 16-byte chunks reads without bank
+// conflicts.  Position of (row r, chunk c in 0..3): line = r >> 1, slot = (((r & 1) << 2) | c) ^ (line & 7).
+
+template <int ELT>
+__device__ __forceinline__ f32x16 mfma_step(const i32x4 (&w)[2], const i32x4 (&x)[2], f32x16 acc);
+
+template <>
+__device__ __forceinline__ f32x16 mfma_step<2>(const i32x4 (&w)[2], const i32x4 (&x)[2], f32x16 acc) {
+  acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, w[0]),
+                                                __builtin_bit_cast(bf16x8, x[0]), acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, w[1]),
+                                                __builtin_bit_cast(bf16x8, x[1]), acc, 0, 0, 0);
+  return acc;
+}
+
+template <>
+__device__ __forceinline__ f32x16 mfma_step<1>(const i32x4 (&w)[2], const i32x4 (&x)[2], f32x16 acc) {
+  i32x8 wa, xa;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    wa[i] = w[0][i];
+    wa[4 + i] = w[1][i];
+    xa[i] = x[0][i];
+    xa[4 + i] = x[1][i];
+  }
+  // cbsz = blgp = 0: both operands e4m3; zero scale operands select the unscaled form (scale 1).
+  return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wa, xa, acc, 0, 0, 0, 0, 0, 0);
+}
+
+template <int ELT>
+__global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmParams p) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  int32_t *s_row_off = reinterpret_cast<int32_t *>(smem + STAGES * STAGE_BYTES);  // [E + 1]
+  int32_t *s_tile_off = s_row_off + (p.nexperts + 1);                             // [E + 1]
+
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: branches on it stay uniform
+  const int lane = tid & 63;
+  const int wn = wave & 3;   // 64-column slice
+  const int wm = wave >> 2;  // 128-row slice == ping-pong group
+  const int tiles_n = (p.n + BN - 1) / BN;
+  const int64_t kbytes = static_cast<int64_t>(p.k) * ELT;
+  const int nk = static_cast<int>(kbytes / KBYTES);
+
+  // ---- schedule tables (exclusive prefix sums over experts) ------------------------------------
+  if (wave == 0) {
+    int row_carry = 0, tile_carry = 0;
+    for (int e0 = 0; e0 < p.nexperts; e0 += 64) {
+      const int e = e0 + lane;
+      int rows = e < p.nexperts ? p.splits[e] : 0;
+      if (rows < 0) rows = 0;
+      const int rows_incl = wave_inclusive_scan(rows);
+      // Rows past max_rows do not exist in A / D: clamp the running offsets.
+      int begin = row_carry + rows_incl - rows;
+      int end = row_carry + rows_incl;
+      if (begin > p.max_rows) begin = p.max_rows;
+      if (end > p.max_rows) end = p.max_rows;
+      const int tiles = ((end - begin + BM - 1) / BM) * tiles_n;
+      const int tiles_incl = wave_inclusive_scan(tiles);
+      if (e < p.nexperts) {
+        s_row_off[e] = begin;
+        s_tile_off[e] = tile_carry + tiles_incl - tiles;
+      }
+      row_carry += __shfl(rows_incl, 63, 64);
+      if (row_carry > p.max_rows) row_carry = p.max_rows;
+      tile_carry += __shfl(tiles_incl, 63, 64);
+    }
+    if (lane == 0) {
+      s_row_off[p.nexperts] = row_carry;
+      s_tile_off[p.nexperts] = tile_carry;
+    }
+  }
+  __syncthreads();
+  const int total_tiles = __builtin_amdgcn_readfirstlane(s_tile_off[p.nexperts]);
+
+  // ---- per-lane constants -----------------------------------------------------------------------
+  // Direct-to-LDS fill: instruction q (0..15) of a tile covers rows [16q, 16q+16); wave w issues
+  // q = 2w and 2w+1.  Lane l lands in line 8q + (l >> 3), slot l & 7, which holds
+  // row 16q + 2*(l >> 3) + (u >> 2), chunk u & 3 with u = (l & 7) ^ (l >> 3).
+  const int fill_u = (lane & 7) ^ (lane >> 3);
+  const int fill_row = 2 * (lane >> 3) + (fill_u >> 2);  // + 16q
+  const int fill_chunk = fill_u & 3;
+  // Fragment reads: lane l reads row (l & 31) of a 32-row block, chunk c(s) for s = 0,1.
+  int frag_off[2];
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    const int c = ELT == 2 ? 2 * s + (lane >> 5) : 2 * (lane >> 5) + s;
+    const int line = (lane & 31) >> 1;
+    const int slot = ((((lane & 1) << 2) | c) ^ (line & 7));
+    frag_off[s] = line * 128 + slot * 16;
+  }
+  const int x_frag_base = wm * 128 * KBYTES;                // rows wm*128.. of the X tile
+  const int w_frag_base = TILE_BYTES + wn * 64 * KBYTES;    // rows wn*64.. of the W tile
+
+  float scalar = p.scalar;
+  if (p.scalar_dev) scalar *= p.scalar_dev[0];
+
+  const int grid = gridDim.x;
+  const int bid = blockIdx.x;
+  // Workgroups are dealt to XCDs round-robin; give each XCD a run of consecutive logical tiles.
+  const int virt = (grid % 8 == 0) ? (bid & 7) * (grid >> 3) + (bid >> 3) : bid;
+
+  int e = 0;
+  for (int tile = virt; tile < total_tiles; tile += grid) {
+    while (tile >= __builtin_amdgcn_readfirstlane(s_tile_off[e + 1])) ++e;
+    const int row_base = __builtin_amdgcn_readfirstlane(s_row_off[e]);
+    const int rows_e = __builtin_amdgcn_readfirstlane(s_row_off[e + 1]) - row_base;
+    const int m_tiles = (rows_e + BM - 1) / BM;
+    const int local = tile - __builtin_amdgcn_readfirstlane(s_tile_off[e]);
+    const int nt = local / m_tiles;
+    const int mt = local - nt * m_tiles;
+    const int m0 = mt * BM;
+    const int n0 = nt * BN;
+
+    // Global source pointers of this lane's 2 + 2 fill instructions (k offset added per step).
+    const uint8_t *xsrc[2];
+    const uint8_t *wsrc[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int r = (2 * wave + j) * 16 + fill_row;
+      int xr = m0 + r;
+      if (xr > rows_e - 1) xr = rows_e - 1;  // tail rows re-read the last valid row
+      int64_t arow = row_base + xr;
+      if (p.gather_a) {
+        arow = p.gather_a[arow];
+        if (p.a_rows > 0) arow = arow < 0 ? 0 : (arow >= p.a_rows ? p.a_rows - 1 : arow);
+      }
+      xsrc[j] = p.a + arow * kbytes + fill_chunk * 16;
+      int wr = n0 + r;
+      if (wr > p.n - 1) wr = p.n - 1;
+      wsrc[j] = p.b + (static_cast<int64_t>(e) * p.n + wr) * kbytes + fill_chunk * 16;
+    }
+
+    auto issue_stage = [&](int kstep) {
+      uint8_t *stage = smem + (kstep % STAGES) * STAGE_BYTES;
+      const int64_t koff = static_cast<int64_t>(kstep) * KBYTES;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        load_to_lds16(xsrc[j] + koff, stage + (2 * wave + j) * 1024);
+        load_to_lds16(wsrc[j] + koff, stage + TILE_BYTES + (2 * wave + j) * 1024);
+      }
+    };
+
+    f32x16 acc[4][2];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+    // ---- prologue: fill DIST stages -------------------------------------------------------------
+    FLUXMI_WAITCNT(0, 0);  // stores of the previous tile's epilogue
+#pragma unroll
+    for (int s = 0; s < DIST; ++s)
+      if (s < nk) issue_stage(s);
+    if (nk >= DIST) {
+      FLUXMI_WAITCNT((DIST - 1) * LOADS_PER_STAGE, 15);
+    } else {
+      FLUXMI_WAITCNT(0, 15);
+    }
+    __builtin_amdgcn_s_barrier();
+    if (wm == 1) __builtin_amdgcn_s_barrier();  // group 1 runs one phase behind group 0
+
+    for (int ks = 0; ks < nk; ++ks) {
+      // ---- memory phase -------------------------------------------------------------------------
+      const uint8_t *stage = smem + (ks % STAGES) * STAGE_BYTES;
+      i32x4 xf[4][2], wf[2][2];
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+          wf[j][s] = *reinterpret_cast<const i32x4 *>(stage + w_frag_base + j * 32 * KBYTES + frag_off[s]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+          xf[i][s] = *reinterpret_cast<const i32x4 *>(stage + x_frag_base + i * 32 * KBYTES + frag_off[s]);
+      if (ks + DIST < nk) {
+        issue_stage(ks + DIST);
+        FLUXMI_WAITCNT((DIST - 1) * LOADS_PER_STAGE, 0);  // stage ks+1 landed, fragments in registers
+      } else {
+        FLUXMI_WAITCNT(0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      // ---- compute phase ------------------------------------------------------------------------
+      __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = mfma_step<ELT>(wf[j], xf[i], acc[i][j]);
+      __builtin_amdgcn_s_setprio(0);
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (wm == 0) __builtin_amdgcn_s_barrier();  // re-align the two groups
+
+    // ---- epilogue: scale, cast, 8-byte stores ---------------------------------------------------
+    const float tile_scale = scalar * (p.alpha ? p.alpha[e] : 1.f);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = m0 + wm * 128 + i * 32 + (lane & 31);
+      if (m >= rows_e) continue;
+      const int64_t srow = row_base + m;
+      const float rs = tile_scale * (p.row_scale ? p.row_scale[srow] : 1.f);
+      int64_t drow = srow;
+      if (p.scatter_d) {
+        drow = p.scatter_d[srow];
+        if (drow < 0 || drow >= p.max_rows) continue;
+      }
+      uint16_t *dptr = p.d + drow * p.n;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int n = n0 + wn * 64 + j * 32 + q * 8 + (lane >> 5) * 4;
+          if (n >= p.n) continue;  // n % 4 == 0 is required, so a quad is all in or all out
+          float v0 = acc[i][j][4 * q + 0] * rs;
+          float v1 = acc[i][j][4 * q + 1] * rs;
+          float v2 = acc[i][j][4 * q + 2] * rs;
+          float v3 = acc[i][j][4 * q + 3] * rs;
+          if (p.col_scale) {
+            const float4 cs =
+                *reinterpret_cast<const float4 *>(p.col_scale + static_cast<int64_t>(e) * p.n + n);
+            v0 *= cs.x;
+            v1 *= cs.y;
+            v2 *= cs.z;
+            v3 *= cs.w;
+          }
+          u32x2 o;
+          o[0] = float_to_bf16_bits(v0) | (static_cast<uint32_t>(float_to_bf16_bits(v1)) << 16);
+          o[1] = float_to_bf16_bits(v2) | (static_cast<uint32_t>(float_to_bf16_bits(v3)) << 16);
+          *reinterpret_cast<u32x2 *>(dptr + n) = o;
+        }
+      }
+    }
+  }
+}
+
+// ---- generic kernel: any K / N, no alignment demands beyond element size -------------------------
+// One thread per output element, a wave covers 64 consecutive columns of one row.  Only used when the
+// MFMA kernel's shape requirements do not hold.
+__device__ __forceinline__ float e4m3_to_float(uint8_t b) {
+  const uint32_t sign = (b & 0x80u) << 24;
+  const uint32_t em = b & 0x7fu;
+  if (em == 0x7fu) return __uint_as_float(sign | 0x7fc00000u);
+  if (em < 8u) return __uint_as_float(sign) + (sign ? -1.f : 1.f) * static_cast<float>(em) * 0x1p-9f;
+  return __uint_as_float(sign | ((em + (120u << 3)) << 20));
+}
+
+template <int ELT>
+__global__ __launch_bounds__(256) void grouped_gemm_generic_kernel(const GemmParams p) {
+  __shared__ int32_t s_row_off[kMaxExperts + 1];
+  if (threadIdx.x == 0) {
+    int acc = 0;
+    for (int e = 0; e < p.nexperts; ++e) {
+      s_row_off[e] = acc;
+      const int v = p.splits[e];
+      acc += v > 0 ? v : 0;
+    }
+    s_row_off[p.nexperts] = acc;
+  }
+  __syncthreads();
+  const int total_rows = s_row_off[p.nexperts] < p.max_rows ? s_row_off[p.nexperts] : p.max_rows;
+  float scalar = p.scalar;
+  if (p.scalar_dev) scalar *= p.scalar_dev[0];
+  const int ncol_blocks = (p.n + 255) / 256;
+  for (int64_t item = blockIdx.x; item < static_cast<int64_t>(total_rows) * ncol_blocks;
+       item += gridDim.x) {
+    const int r = static_cast<int>(item / ncol_blocks);
+    const int n = static_cast<int>(item % ncol_blocks) * 256 + threadIdx.x;
+    int e = 0;
+    while (r >= s_row_off[e + 1]) ++e;
+    if (n >= p.n) continue;
+    int64_t arow = r;
+    if (p.gather_a) {
+      arow = p.gather_a[r];
+      if (p.a_rows > 0) arow = arow < 0 ? 0 : (arow >= p.a_rows ? p.a_rows - 1 : arow);
+    }
+    const uint8_t *ap = p.a + arow * p.k * ELT;
+    const uint8_t *bp = p.b + (static_cast<int64_t>(e) * p.n + n) * p.k * ELT;
+    float acc = 0.f;
+    for (int kk = 0; kk < p.k; ++kk) {
+      float av, bv;
+      if (ELT == 2) {
+        av = bf16_bits_to_float(reinterpret_cast<const uint16_t *>(ap)[kk]);
+        bv = bf16_bits_to_float(reinterpret_cast<const uint16_t *>(bp)[kk]);
+      } else {
+        av = e4m3_to_float(ap[kk]);
+        bv = e4m3_to_float(bp[kk]);
+      }
+      acc = fmaf(av, bv, acc);
+    }
+    float v = acc * scalar * (p.alpha ? p.alpha[e] : 1.f) * (p.row_scale ? p.row_scale[r] : 1.f);
+    if (p.col_scale) v *= p.col_scale[static_cast<int64_t>(e) * p.n + n];
+    int64_t drow = r;
+    if (p.scatter_d) {
+      drow = p.scatter_d[r];
+      if (drow < 0 || drow >= p.max_rows) continue;
+    }
+    p.d[drow * p.n + n] = float_to_bf16_bits(v);
+  }
+}
+
+bool mfma_path_ok(const fluxmi_grouped_gemm_args *a) {
+  const int elt = a->dtype == FLUXMI_BF16 ? 2 : 1;
+  const int64_t kbytes = static_cast<int64_t>(a->k) * elt;
+  return kbytes % KBYTES == 0 && kbytes >= KBYTES && a->n % 4 == 0 && aligned16(a->a) &&
+         aligned16(a->b) && (reinterpret_cast<uintptr_t>(a->d) & 7u) == 0 &&
+         (a->col_scale == nullptr || aligned16(a->col_scale));
+}
+
+size_t mfma_lds_bytes(int nexperts) {
+  return static_cast<size_t>(STAGES) * STAGE_BYTES + 2 * static_cast<size_t>(nexperts + 1) * sizeof(int32_t);
+}
+
+}  // namespace
+}  // namespace fluxmi
+
+extern "C" size_t fluxmi_grouped_gemm_workspace_bytes(const fluxmi_grouped_gemm_args *) { return 0; }
+
+extern "C" int fluxmi_grouped_gemm(const fluxmi_grouped_gemm_args *args, void *, size_t, void *stream) {
+  using namespace fluxmi;
+  FLUXMI_REQUIRE(args != nullptr, FLUXMI_ERR_INVALID_ARG, "grouped_gemm: null args");
+  FLUXMI_REQUIRE(args->dtype == FLUXMI_BF16 || args->dtype == FLUXMI_FP8_E4M3, FLUXMI_ERR_INVALID_ARG,
+                 "grouped_gemm: unknown dtype %d", args->dtype);
+  FLUXMI_REQUIRE(args->reserved1 == 0, FLUXMI_ERR_INVALID_ARG, "grouped_gemm: reserved field must be 0");
+  FLUXMI_REQUIRE(args->a_rows >= 0, FLUXMI_ERR_INVALID_ARG, "grouped_gemm: negative a_rows");
+  FLUXMI_REQUIRE(args->nexperts >= 1 && args->nexperts <= kMaxExperts, FLUXMI_ERR_UNSUPPORTED,
+                 "grouped_gemm: nexperts=%d outside [1,%d]", args->nexperts, kMaxExperts);
+  FLUXMI_REQUIRE(args->max_rows >= 0 && args->n >= 0 && args->k >= 0, FLUXMI_ERR_INVALID_ARG,
+                 "grouped_gemm: negative size (max_rows=%d, n=%d, k=%d)", args->max_rows, args->n,
+                 args->k);
+  if (args->max_rows == 0 || args->n == 0) return FLUXMI_OK;
+  FLUXMI_REQUIRE(args->k >= 1, FLUXMI_ERR_UNSUPPORTED, "grouped_gemm: k must be positive");
+  FLUXMI_REQUIRE(args->a && args->b && args->d && args->splits, FLUXMI_ERR_INVALID_ARG,
+                 "grouped_gemm: null a / b / d / splits");
+
+  GemmParams p;
+  p.a = static_cast<const uint8_t *>(args->a);
+  p.b = static_cast<const uint8_t *>(args->b);
+  p.d = static_cast<uint16_t *>(args->d);
+  p.splits = args->splits;
+  p.gather_a = args->gather_a;
+  p.scatter_d = args->scatter_d;
+  p.alpha = args->alpha;
+  p.row_scale = args->row_scale;
+  p.col_scale = args->col_scale;
+  p.scalar_dev = args->scalar_scale_dev;
+  p.scalar = args->scalar_scale;
+  p.nexperts = args->nexperts;
+  p.max_rows = args->max_rows;
+  p.a_rows = args->a_rows;
+  p.n = args->n;
+  p.k = args->k;
+
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int cus = fluxmi_device_cu_count();
+  FLUXMI_REQUIRE(cus > 0, FLUXMI_ERR_HIP, "grouped_gemm: cannot query the device");
+
+  if (mfma_path_ok(args)) {
+    const size_t lds = mfma_lds_bytes(args->nexperts);
+    // Upper bound of the tile count: never launch more workgroups than tiles.
+    const int64_t tiles_n = (args->n + BN - 1) / BN;
+    const int64_t max_tiles = (static_cast<int64_t>(args->max_rows) / BM + args->nexperts) * tiles_n;
+    const int grid = static_cast<int>(max_tiles < cus ? max_tiles : cus);
+    if (args->dtype == FLUXMI_BF16) {
+      static bool attr_set = false;
+      if (!attr_set) {
+        FLUXMI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(grouped_gemm_mfma_kernel<2>),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        attr_set = true;
+      }
+      hipLaunchKernelGGL(grouped_gemm_mfma_kernel<2>, dim3(grid), dim3(NTHREADS), lds, s, p);
+    } else {
+      static bool attr_set = false;
+      if (!attr_set) {
+        FLUXMI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(grouped_gemm_mfma_kernel<1>),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        attr_set = true;
+      }
+      hipLaunchKernelGGL(grouped_gemm_mfma_kernel<1>, dim3(grid), dim3(NTHREADS), lds, s, p);
+    }
+  } else {
+    const int grid = cus * 8;
+    if (args->dtype == FLUXMI_BF16)
+      hipLaunchKernelGGL(grouped_gemm_generic_kernel<2>, dim3(grid), dim3(256), 0, s, p);
+    else
+      hipLaunchKernelGGL(grouped_gemm_generic_kernel<1>, dim3(grid), dim3(256), 0, s, p);
+  }
+  FLUXMI_HIP_CHECK(hipGetLastError());
+  return FLUXMI_OK;
+}

@@ -1,0 +1,223 @@
+// Routing: stable counting sort of (token, k) pairs by expert id -> splits, offsets, scatter_index,
+// gather_index, topk_index.
+//
+// The flat pair array is cut into chunks of kChunk = 512 pairs, one wave per chunk (8 wave-steps of 64).
+//   1. route_hist_kernel    per-chunk expert histogram in LDS (ds_add_u32), written to hist[chunk][e]
+//   2. route_scan_kernel    one wave per expert: exclusive scan of hist[:, e] over chunks (wave scan),
+//                           in place; the total is splits[e]
+//   3. route_scatter_kernel per chunk: running[e] = offsets[e] + base[chunk][e] in LDS; for each
+//                           wave-step the lanes holding the same expert are found with ballots over the
+//                           bits of the id, ranked with mbcnt, and the first of them advances running[e].
+// Every pair is read twice (8 B) and each output written once: the array traffic is the whole cost.
+#include "common.hpp"
+
+namespace fluxmi {
+namespace {
+
+constexpr int kChunk = 512;           // pairs per wave
+constexpr int kWavesPerBlock = 4;
+constexpr int kThreads = kWavesPerBlock * 64;
+constexpr int kMaxExperts = 1024;
+
+__global__ __launch_bounds__(kThreads) void route_hist_kernel(const int32_t *__restrict__ choosed,
+                                                              int32_t npairs, int32_t nexperts,
+                                                              int32_t nchunks,
+                                                              int32_t *__restrict__ hist) {
+  extern __shared__ int32_t s_hist[];  // [kWavesPerBlock][nexperts]
+  const int wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  for (int i = threadIdx.x; i < kWavesPerBlock * nexperts; i += kThreads) s_hist[i] = 0;
+  __syncthreads();
+  const int chunk = blockIdx.x * kWavesPerBlock + wave;
+  int32_t *my = s_hist + wave * nexperts;
+  if (chunk < nchunks) {
+    const int base = chunk * kChunk;
+#pragma unroll
+    for (int s = 0; s < kChunk / 64; ++s) {
+      const int i = base + s * 64 + lane;
+      if (i < npairs) {
+        const int32_t e = choosed[i];
+        if (e >= 0 && e < nexperts) atomicAdd(&my[e], 1);
+      }
+    }
+  }
+  __syncthreads();
+  if (chunk < nchunks) {
+    for (int e = lane; e < nexperts; e += 64) hist[static_cast<size_t>(chunk) * nexperts + e] = my[e];
+  }
+}
+
+// grid = ceil(E / 4) blocks of 4 waves; wave -> expert.
+__global__ __launch_bounds__(kThreads) void route_scan_kernel(int32_t *__restrict__ hist,
+                                                              int32_t nexperts, int32_t nchunks,
+                                                              int32_t *__restrict__ splits_ws,
+                                                              int32_t *__restrict__ splits_out) {
+  const int e = blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (e >= nexperts) return;
+  int running = 0;
+  for (int c0 = 0; c0 < nchunks; c0 += 64) {
+    const int c = c0 + lane;
+    const int v = c < nchunks ? hist[static_cast<size_t>(c) * nexperts + e] : 0;
+    const int incl = wave_inclusive_scan(v);
+    if (c < nchunks) hist[static_cast<size_t>(c) * nexperts + e] = running + incl - v;
+    running += __shfl(incl, 63, 64);
+  }
+  if (lane == 0) {
+    splits_ws[e] = running;
+    if (splits_out) splits_out[e] = running;
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void route_scatter_kernel(
+    const int32_t *__restrict__ choosed, int32_t npairs, int32_t topk, int32_t nexperts,
+    int32_t nchunks, int32_t idbits, const int32_t *__restrict__ base,
+    const int32_t *__restrict__ splits_ws, int32_t *__restrict__ offsets_out,
+    int32_t *__restrict__ scatter_index, int32_t *__restrict__ gather_index,
+    int32_t *__restrict__ topk_index) {
+  extern __shared__ int32_t s_mem[];  // [nexperts] offsets, then [kWavesPerBlock][nexperts] running
+  int32_t *s_off = s_mem;
+  const int wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  int32_t *running = s_mem + nexperts + wave * nexperts;
+
+  // Exclusive prefix sum of splits -> offsets (every block recomputes it; E <= 1024).
+  if (wave == 0) {
+    int carry = 0;
+    for (int e0 = 0; e0 < nexperts; e0 += 64) {
+      const int e = e0 + lane;
+      const int v = e < nexperts ? splits_ws[e] : 0;
+      const int incl = wave_inclusive_scan(v);
+      if (e < nexperts) s_off[e] = carry + incl - v;
+      carry += __shfl(incl, 63, 64);
+    }
+    if (blockIdx.x == 0 && offsets_out) {
+      for (int e = lane; e < nexperts; e += 64) offsets_out[e] = s_off[e];
+      if (lane == 0) offsets_out[nexperts] = carry;
+    }
+  }
+  __syncthreads();
+
+  const int chunk = blockIdx.x * kWavesPerBlock + wave;
+  if (chunk >= nchunks) return;
+  for (int e = lane; e < nexperts; e += 64)
+    running[e] = s_off[e] + base[static_cast<size_t>(chunk) * nexperts + e];
+  __builtin_amdgcn_wave_barrier();
+
+  const int first = chunk * kChunk;
+  for (int s = 0; s < kChunk / 64; ++s) {
+    const int i = first + s * 64 + lane;
+    int32_t e = -1;
+    if (i < npairs) {
+      e = choosed[i];
+      if (e < 0 || e >= nexperts) e = -1;
+    }
+    // Lanes that hold the same expert id as this lane.
+    uint64_t same = __ballot(e >= 0);
+    for (int b = 0; b < idbits; ++b) {
+      const uint64_t bit = __ballot((e >> b) & 1);
+      same &= ((e >> b) & 1) ? bit : ~bit;
+    }
+    if (e >= 0) {
+      const int rank = popc_below_lane(same);
+      const int start = running[e];
+      __builtin_amdgcn_wave_barrier();
+      if (rank == 0) running[e] = start + __popcll(same);
+      const int row = start + rank;
+      scatter_index[i] = row;
+      if (gather_index) gather_index[row] = i / topk;
+      if (topk_index) topk_index[row] = i % topk;
+    } else {
+      __builtin_amdgcn_wave_barrier();
+      if (i < npairs) scatter_index[i] = -1;
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
+__global__ __launch_bounds__(256) void gather_index_kernel(const int32_t *__restrict__ scatter_index,
+                                                           int32_t npairs, int32_t nrows,
+                                                           int32_t topk,
+                                                           int32_t *__restrict__ gather_index,
+                                                           int32_t *__restrict__ topk_index) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= npairs) return;
+  const int32_t row = scatter_index[i];
+  if (row < 0 || row >= nrows) return;
+  gather_index[row] = i / topk;
+  if (topk_index) topk_index[row] = i % topk;
+}
+
+inline int32_t num_chunks(int64_t npairs) { return static_cast<int32_t>((npairs + kChunk - 1) / kChunk); }
+
+}  // namespace
+}  // namespace fluxmi
+
+extern "C" size_t fluxmi_moe_route_sort_workspace_bytes(int32_t ntokens, int32_t topk,
+                                                        int32_t nexperts) {
+  using namespace fluxmi;
+  if (ntokens < 0 || topk < 1 || nexperts < 1) return 0;
+  const int64_t npairs = static_cast<int64_t>(ntokens) * topk;
+  const int64_t nchunks = num_chunks(npairs) > 0 ? num_chunks(npairs) : 1;
+  return static_cast<size_t>((nchunks + 1) * nexperts) * sizeof(int32_t);
+}
+
+extern "C" int fluxmi_moe_route_sort(const int32_t *choosed, int32_t ntokens, int32_t topk,
+                                     int32_t nexperts, int32_t *splits, int32_t *offsets,
+                                     int32_t *scatter_index, int32_t *gather_index,
+                                     int32_t *topk_index, void *workspace, size_t workspace_bytes,
+                                     void *stream) {
+  using namespace fluxmi;
+  FLUXMI_REQUIRE(ntokens >= 0 && topk >= 1, FLUXMI_ERR_INVALID_ARG,
+                 "moe_route_sort: bad sizes (ntokens=%d, topk=%d)", ntokens, topk);
+  FLUXMI_REQUIRE(nexperts >= 1 && nexperts <= kMaxExperts, FLUXMI_ERR_UNSUPPORTED,
+                 "moe_route_sort: nexperts=%d outside [1,%d]", nexperts, kMaxExperts);
+  const int64_t npairs64 = static_cast<int64_t>(ntokens) * topk;
+  FLUXMI_REQUIRE(npairs64 <= (int64_t{1} << 30), FLUXMI_ERR_UNSUPPORTED,
+                 "moe_route_sort: ntokens*topk=%lld exceeds 2^30", static_cast<long long>(npairs64));
+  FLUXMI_REQUIRE(scatter_index != nullptr && (choosed != nullptr || npairs64 == 0),
+                 FLUXMI_ERR_INVALID_ARG, "moe_route_sort: null choosed / scatter_index");
+  const size_t need = fluxmi_moe_route_sort_workspace_bytes(ntokens, topk, nexperts);
+  FLUXMI_REQUIRE(workspace != nullptr && workspace_bytes >= need, FLUXMI_ERR_WORKSPACE,
+                 "moe_route_sort: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+  const int32_t npairs = static_cast<int32_t>(npairs64);
+  const int32_t nchunks = num_chunks(npairs);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  int32_t *splits_ws = static_cast<int32_t *>(workspace);
+  int32_t *hist = splits_ws + nexperts;
+  int idbits = 0;
+  while ((1 << idbits) < nexperts) ++idbits;
+
+  const unsigned nblocks = static_cast<unsigned>((nchunks + kWavesPerBlock - 1) / kWavesPerBlock);
+  if (nchunks > 0) {
+    hipLaunchKernelGGL(route_hist_kernel, dim3(nblocks), dim3(kThreads),
+                       kWavesPerBlock * nexperts * sizeof(int32_t), s, choosed, npairs, nexperts,
+                       nchunks, hist);
+  }
+  hipLaunchKernelGGL(route_scan_kernel, dim3((nexperts + kWavesPerBlock - 1) / kWavesPerBlock),
+                     dim3(kThreads), 0, s, hist, nexperts, nchunks, splits_ws, splits);
+  // With no pairs one block still runs to publish offsets (all zero).
+  hipLaunchKernelGGL(route_scatter_kernel, dim3(nblocks > 0 ? nblocks : 1), dim3(kThreads),
+                     (1 + kWavesPerBlock) * nexperts * sizeof(int32_t), s, choosed, npairs, topk,
+                     nexperts, nchunks, idbits, hist, splits_ws, offsets, scatter_index, gather_index,
+                     topk_index);
+  FLUXMI_HIP_CHECK(hipGetLastError());
+  return FLUXMI_OK;
+}
+
+extern "C" int fluxmi_moe_gather_index(const int32_t *scatter_index, int32_t nrows, int32_t topk,
+                                       int32_t *gather_index, int32_t *topk_index, void *stream) {
+  using namespace fluxmi;
+  FLUXMI_REQUIRE(nrows >= 0 && topk >= 1, FLUXMI_ERR_INVALID_ARG,
+                 "moe_gather_index: bad sizes (nrows=%d, topk=%d)", nrows, topk);
+  FLUXMI_REQUIRE(nrows % topk == 0, FLUXMI_ERR_INVALID_ARG,
+                 "moe_gather_index: nrows=%d is not a multiple of topk=%d", nrows, topk);
+  if (nrows == 0) return FLUXMI_OK;
+  FLUXMI_REQUIRE(scatter_index != nullptr && gather_index != nullptr, FLUXMI_ERR_INVALID_ARG,
+                 "moe_gather_index: null pointer argument");
+  hipLaunchKernelGGL(gather_index_kernel, dim3((nrows + 255) / 256), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), scatter_index, nrows, nrows, topk, gather_index,
+                     topk_index);
+  FLUXMI_HIP_CHECK(hipGetLastError());
+  return FLUXMI_OK;
+}

@@ -1,0 +1,155 @@
+/*
+ * fluxmi.h — C-ABI of the MI355X (gfx950) kernels behind Flux's single-GPU MoE operators.
+ *
+ * Every entry point takes plain device pointers, sizes and a HIP stream (passed as `void*`, i.e. a
+ * `hipStream_t`; NULL = the default stream).  Nothing here allocates device memory: scratch space is
+ * caller-provided (`workspace`, sized by the matching `*_workspace_bytes` call).  All calls are
+ * asynchronous with respect to the host and never synchronise the stream.  Return value: 0 on success,
+ * a negative `fluxmi_status` otherwise; `fluxmi_last_error()` gives a thread-local message.
+ *
+ * Citations name the interface of the reference (bytedance/flux) that each entry point stands in for.
+ */
+#ifndef FLUXMI_H_
+#define FLUXMI_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum fluxmi_status {
+  FLUXMI_OK = 0,
+  FLUXMI_ERR_INVALID_ARG = -1, /* null pointer, negative size, misaligned pointer, bad enum */
+  FLUXMI_ERR_UNSUPPORTED = -2, /* shape / dtype combination no kernel covers */
+  FLUXMI_ERR_WORKSPACE = -3,   /* workspace missing or too small */
+  FLUXMI_ERR_HIP = -4          /* a HIP runtime call or kernel launch failed */
+} fluxmi_status;
+
+typedef enum fluxmi_dtype {
+  FLUXMI_BF16 = 0,    /* bfloat16 operands, fp32 accumulate */
+  FLUXMI_FP8_E4M3 = 1 /* OCP e4m3 (torch.float8_e4m3fn) operands, fp32 accumulate */
+} fluxmi_dtype;
+
+/* Library version (major*10000 + minor*100 + patch) and the last error text of the calling thread. */
+int fluxmi_version(void);
+const char *fluxmi_last_error(void);
+
+/* Number of compute units of the current device (persistent kernels launch one workgroup per CU). */
+int fluxmi_device_cu_count(void);
+
+/* ------------------------------------------------------------------------------------------------
+ * Routing: stable counting sort of (token, k) pairs by expert id.
+ *
+ * Stands in for `torch.bincount` + `calc_scatter_index_stable` + `calc_gather_index`
+ * (python/flux/testing/moe_utils.py:141-144, :96-138, :215-217) and for the device kernels
+ * `calc_scatter_index` (src/cuda/moe_utils.cu:23-75) and `calc_gather_index_impl`
+ * (src/moe_ag_scatter/sort_util.cu:39-92, :121-160), with the *stable* order as the contract:
+ *   splits[e]          = #{i : choosed[i] == e}
+ *   offsets            = exclusive prefix sum of splits, offsets[E] = number of routed pairs
+ *   scatter_index[i]   = offsets[choosed[i]] + #{i' < i : choosed[i'] == choosed[i]}
+ *   gather_index[scatter_index[i]] = i / topk,   topk_index[scatter_index[i]] = i % topk
+ * `choosed` holds ntokens*topk int32 in [0, nexperts); ids outside that range are treated as dropped
+ * pairs: they get scatter_index -1 and take no row.  Any of the output pointers except
+ * `scatter_index` may be NULL.
+ * ---------------------------------------------------------------------------------------------- */
+size_t fluxmi_moe_route_sort_workspace_bytes(int32_t ntokens, int32_t topk, int32_t nexperts);
+int fluxmi_moe_route_sort(const int32_t *choosed, int32_t ntokens, int32_t topk, int32_t nexperts,
+                          int32_t *splits, int32_t *offsets, int32_t *scatter_index,
+                          int32_t *gather_index, int32_t *topk_index, void *workspace,
+                          size_t workspace_bytes, void *stream);
+
+/* Inverse permutation only: `calc_gather_index_impl` (src/moe_ag_scatter/sort_util.cu:121-160).
+ * gather_index[scatter_index[i]] = i / topk, topk_index[...] = i % topk for scatter_index[i] in
+ * [0, nrows); entries outside are skipped.  topk_index may be NULL. */
+int fluxmi_moe_gather_index(const int32_t *scatter_index, int32_t nrows, int32_t topk,
+                            int32_t *gather_index, int32_t *topk_index, void *stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Grouped GEMM over ragged per-expert row counts (layer0 and the GEMM half of layer1).
+ *
+ * Stands in for the kernels behind `GemmGroupedV3AGScatterOp::forward_impl`
+ * (src/moe_ag_scatter/ths_op/gemm_grouped_v3_ag_scatter.cc:227-447, arguments
+ * include/flux/args/moe_ag_scatter.h:25-35) and the GEMM part of `GemmGroupedV3GatherRS`
+ * (src/moe_gather_rs/ths_op/gemm_grouped_v3_gather_rs.cc:245-537, include/flux/args/moe_gather_rs.h:78-117)
+ * and the plain `GemmGroupedV3` (src/comm_none/ths_op/gemm_grouped_v3.cc:43-171):
+ *
+ *   for sorted row r of expert e (offsets[e] <= r < offsets[e+1], offsets = prefix sum of splits):
+ *     acc[n]   = sum_k float(A[gather_a ? gather_a[r] : r, k]) * float(B[e, n, k])        (fp32)
+ *     D[scatter_d ? scatter_d[r] : r, n] =
+ *         bf16( acc[n] * (alpha ? alpha[e] : 1) * (row_scale ? row_scale[r] : 1)
+ *                      * (col_scale ? col_scale[e*N + n] : 1) * scalar_scale )
+ *
+ * A is row-major [*, K] (lda = K), B is [E, N, K] with K contiguous, D is row-major [*, N] bf16.
+ * `splits` is a DEVICE int32 array of `nexperts` row counts; the tile schedule is derived from it on
+ * the device, so the host never reads it.  `max_rows` is an upper bound of sum(splits) (ntokens*topk);
+ * rows beyond sum(splits) are not touched.  Requirements: K % 64 == 0 (bf16) or K % 128 == 0 (fp8)
+ * for the MFMA kernels — other K take a slower generic kernel; pointers 16-byte aligned.
+ * ---------------------------------------------------------------------------------------------- */
+typedef struct fluxmi_grouped_gemm_args {
+  int32_t dtype;         /* fluxmi_dtype of A and B */
+  int32_t nexperts;      /* E */
+  int32_t max_rows;      /* upper bound on the number of sorted rows */
+  int32_t n;             /* N, columns of D / rows of each B[e] */
+  int32_t k;             /* K */
+  int32_t a_rows;        /* rows of A when gather_a is given: entries are clamped into [0, a_rows); 0 = trust them */
+  const void *a;         /* [rows_a, K] */
+  const void *b;         /* [E, N, K] */
+  void *d;               /* [max_rows, N] bf16 */
+  const int32_t *splits; /* device [E] */
+  const int32_t *gather_a;  /* device [max_rows] or NULL */
+  const int32_t *scatter_d; /* device [max_rows] or NULL */
+  const float *alpha;       /* device [E] or NULL  (Flux `output_scale` / `weight_scale`) */
+  const float *row_scale;   /* device [max_rows] or NULL, indexed by sorted row */
+  const float *col_scale;   /* device [E, N] or NULL */
+  float scalar_scale;       /* host scalar, 1.0f for none (Flux `input_scale[0]` is passed by pointer below) */
+  int32_t reserved1;        /* must be 0 */
+  const float *scalar_scale_dev; /* device [1] or NULL; multiplied in if given */
+} fluxmi_grouped_gemm_args;
+
+size_t fluxmi_grouped_gemm_workspace_bytes(const fluxmi_grouped_gemm_args *args);
+int fluxmi_grouped_gemm(const fluxmi_grouped_gemm_args *args, void *workspace,
+                        size_t workspace_bytes, void *stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Top-k (weighted) gather-reduce back to token order (the reduce half of layer1).
+ *
+ * Stands in for `topk_reduce_scatter_impl` behind `flux.topk_scatter_reduce`
+ * (src/moe_gather_rs/moe_utils.cu:282-395, src/moe_gather_rs/ths_op/topk_scatter_reduce.cc:30-56), the
+ * reduce part of the fused layer1 kernel (src/moe_gather_rs/sm90_gemm_array_threadblock_specialized.hpp:1306-1409)
+ * and its weighted form (src/moe_gather_rs/topk_gather_rs_v2.cu:394-407):
+ *
+ *   out[t, n] = bf16( scale * sum_{g < ngroups} sum_{j < topk}
+ *                       w[r] * float(in[g][r, n]) ),   r = routing_idx[t*topk + j],
+ *   w[r] = row_weight ? row_weight[r] : 1;  rows with r < 0 are skipped; fp32 accumulation in the
+ *   order g-major then j; one rounding at the end.
+ * `in` is an array (on the HOST) of `ngroups` device pointers to row-major bf16 [nrows, n] matrices.
+ * Requirements: n % 8 == 0, 1 <= ngroups <= 4, 1 <= topk <= 64.
+ * ---------------------------------------------------------------------------------------------- */
+int fluxmi_topk_gather_reduce(const void *const *in, int32_t ngroups, const int32_t *routing_idx,
+                              const float *row_weight, float scale, int32_t ntokens, int32_t topk,
+                              int32_t n, void *out, void *stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * bf16 -> fp8-e4m3 absmax quantisation, one scale per (row, block of `block_cols` columns).
+ *
+ * Stands in for `block_scaled_1d_cast_transpose_impl` behind `Quantization::quantize_vector_blockwise`
+ * (src/quantization/quantization.cu:306-367, :421-706, :1382-1456; src/quantization/ths_op/quantization.cc:75-145):
+ *   amax  = max |float(x)| over the block,  a = max(amax, eps)
+ *   scale = 1 if a == 0; 448 / a (fp32 division); if that is +inf, 0x1.FEp127
+ *   q     = e4m3_round_nearest_even_saturate( float(x) * scale )
+ *   scale_inv = float(1.0 / double(scale))
+ * block_cols == 0 means one block per row (per-token scale, scale_inv is [rows]); block_cols == 128 is
+ * Flux's 1x128 form.  With `permute_scale` != 0 and block_cols == 128 scale_inv is stored as
+ * [ceil(rows/128), ceil(cols/128), 128] (row-in-block fastest), otherwise as [rows, nblocks].
+ * Requirements: cols % 8 == 0.
+ * ---------------------------------------------------------------------------------------------- */
+int fluxmi_quant_e4m3_rowwise(const void *x_bf16, int64_t rows, int64_t cols, int32_t block_cols,
+                              float eps, void *q_out, float *scale_inv_out, int32_t permute_scale,
+                              void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLUXMI_H_ */

@@ -1,0 +1,220 @@
+"""GPU parity, grouped GEMM (bf16 and fp8): bf16 outputs within rtol 1e-2 / atol 1e-2 of the fp32-accumulated
+oracle; fp8 outputs within 3e-2 relative Frobenius error of the dequantise-matmul oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import configs, layers, quant, routing
+
+pytestmark = pytest.mark.gpu
+RTOL, ATOL = 1e-2, 1e-2
+FP8_FROB = 3e-2
+
+
+def assert_close(got_bf16, ref_f32, what=""):
+    got = got_bf16.float().cpu()
+    bad = (got - ref_f32).abs() > ATOL + RTOL * ref_f32.abs()
+    assert not bool(bad.any()), f"{what}: {int(bad.sum())} of {bad.numel()} outside tolerance, max err " \
+                                f"{float((got - ref_f32).abs().max())}"
+
+
+def random_splits(rng, experts, rows, empty=()):
+    p = rng.random(experts) + 0.05
+    for e in empty:
+        p[e] = 0
+    cnt = rng.multinomial(rows, p / p.sum())
+    return cnt.astype(np.int32)
+
+
+@pytest.mark.parametrize("experts,rows,n,k,seed,empty", [
+    (1, 256, 256, 64, 0, ()), (1, 300, 264, 128, 1, ()), (4, 1000, 512, 256, 2, ()), (8, 2048, 1024, 1024, 3, (0, 5)),
+    (3, 700, 1408, 2048, 4, (1,)), (16, 900, 256, 320, 5, (2, 3, 15)), (2, 17, 8, 32, 6, ()), (5, 1, 512, 64, 7, (0, 1, 2, 4)),
+    (64, 6000, 384, 512, 8, ())])
+def test_bf16_plain_against_oracle(experts, rows, n, k, seed, empty):
+    from flux_amd import capi
+    print(f"[case] grouped_gemm bf16 E={experts} rows={rows} N={n} K={k} empty={empty}", flush=True)
+    rng = np.random.default_rng(seed)
+    g = torch.Generator().manual_seed(seed)
+    split = random_splits(rng, experts, rows, empty)
+    a = torch.randn(rows, k, generator=g).to(torch.bfloat16)
+    w = (torch.randn(experts, n, k, generator=g) * 0.05).to(torch.bfloat16)
+    ref = layers.grouped_gemm_fp32(a, w, split)
+    out = capi.grouped_gemm(a.cuda(), w.cuda(), torch.from_numpy(split).cuda())
+    assert_close(out, ref, "plain")
+
+
+def test_bf16_gather_scatter_and_scales():
+    from flux_amd import capi
+    rng = np.random.default_rng(21)
+    g = torch.Generator().manual_seed(21)
+    tokens, topk, experts, h, n = 300, 3, 6, 256, 520
+    choosed = np.stack([rng.permutation(experts)[:topk] for _ in range(tokens)]).astype(np.int32)
+    split = routing.splits(choosed, experts)
+    si = routing.scatter_index_stable(choosed, experts)
+    gi, _ = routing.gather_index(si, topk)
+    m = tokens * topk
+    x = torch.randn(tokens, h, generator=g).to(torch.bfloat16)
+    w = (torch.randn(experts, n, h, generator=g) * 0.05).to(torch.bfloat16)
+    alpha = torch.rand(experts, generator=g) + 0.5
+    rs = torch.rand(m, generator=g) + 0.5
+    cs = torch.rand(experts, n, generator=g) + 0.5
+    sdev = torch.tensor([1.5])
+    perm = torch.randperm(m, generator=g).to(torch.int32)
+    xs = x[torch.as_tensor(gi, dtype=torch.long)]
+    ref = layers.grouped_gemm_fp32(xs, w, split, alpha=alpha, row_scale=rs, col_scale=cs, scalar=0.5 * 1.5)
+    ref_scattered = torch.zeros_like(ref)
+    ref_scattered[perm.long()] = ref
+    out = capi.grouped_gemm(x.cuda(), w.cuda(), torch.from_numpy(split).cuda(), gather_a=torch.from_numpy(gi).cuda(),
+                            scatter_d=perm.cuda(), alpha=alpha.cuda(), row_scale=rs.cuda(), col_scale=cs.cuda(),
+                            scalar_scale=0.5, scalar_scale_dev=sdev.cuda())
+    assert_close(out, ref_scattered, "gather+scatter+scales")
+
+
+def test_bf16_generic_kernel_odd_shapes():
+    """K not a multiple of 32 and N not a multiple of 4 take the generic kernel."""
+    from flux_amd import capi
+    g = torch.Generator().manual_seed(31)
+    split = np.array([13, 0, 20], dtype=np.int32)
+    a = torch.randn(33, 72, generator=g).to(torch.bfloat16)
+    w = (torch.randn(3, 50, 72, generator=g) * 0.1).to(torch.bfloat16)
+    ref = layers.grouped_gemm_fp32(a, w, split)
+    out = capi.grouped_gemm(a.cuda(), w.cuda(), torch.from_numpy(split).cuda())
+    assert_close(out, ref, "generic")
+
+
+def test_rows_beyond_splits_untouched():
+    from flux_amd import capi
+    g = torch.Generator().manual_seed(41)
+    split = np.array([100, 50], dtype=np.int32)
+    a = torch.randn(400, 64, generator=g).to(torch.bfloat16)
+    w = (torch.randn(2, 256, 64, generator=g) * 0.1).to(torch.bfloat16)
+    out = torch.full((400, 256), 7.0, dtype=torch.bfloat16, device="cuda")
+    capi.grouped_gemm(a.cuda(), w.cuda(), torch.from_numpy(split).cuda(), out=out)
+    ref = layers.grouped_gemm_fp32(a[:150], w, split)
+    assert_close(out[:150], ref, "rows")
+    assert bool((out[150:] == 7.0).all())
+
+
+def test_single_expert_matches_dense_gemm():
+    """E = 1 reduces to one dense GEMM: cross-check with torch.mm (hipBLASLt) on the GPU."""
+    from flux_amd import capi
+    gen = torch.Generator(device="cuda").manual_seed(51)
+    a = torch.randn(1024, 2048, generator=gen, device="cuda").to(torch.bfloat16)
+    w = (torch.randn(1, 768, 2048, generator=gen, device="cuda") * 0.02).to(torch.bfloat16)
+    out = capi.grouped_gemm(a, w, torch.tensor([1024], dtype=torch.int32, device="cuda"))
+    ref = (a.float() @ w[0].float().t()).cpu()
+    assert_close(out, ref, "dense")
+
+
+def sampled_rows(split, per_expert, rng):
+    off = routing.offsets(split)
+    rows = []
+    for e in range(len(split)):
+        lo, hi = int(off[e]), int(off[e + 1])
+        if hi == lo:
+            continue
+        pick = {lo, hi - 1, lo + (hi - lo) // 2}
+        pick.update(int(v) for v in rng.integers(lo, hi, size=per_expert))
+        rows.extend(sorted(pick))
+    return np.array(rows, dtype=np.int64)
+
+
+@pytest.mark.parametrize("name", ["C1", "C2", "C3", "C4"])
+def test_benchmark_layer0_and_layer1(name):
+    """The benchmark shapes at full size.  C1 is compared in full; the larger ones on a sample of sorted rows per
+    expert (first, last, middle and random rows, all columns) computed by the oracle in fp32."""
+    from flux_amd import capi
+    wl = configs.make_workload(name, with_w2=(name != "C2"))
+    print(f"[case] grouped_gemm {name} M={wl.rows} H={wl.hidden} F={wl.ffn} E={wl.experts}", flush=True)
+    rng = np.random.default_rng(61)
+    x, w1 = wl.tensors["x"], wl.tensors["w1"]
+    split_d = torch.from_numpy(wl.splits).cuda()
+    gi_d = torch.from_numpy(wl.gather_index).cuda()
+    out0 = capi.grouped_gemm(x.cuda(), w1.cuda(), split_d, gather_a=gi_d)
+    eor = routing.expert_of_row(wl.splits)
+    rows = np.arange(wl.rows) if name == "C1" else sampled_rows(wl.splits, 6 if name == "C4" else 24, rng)
+    for e in np.unique(eor[rows]):
+        r = rows[eor[rows] == e]
+        ref = x[torch.as_tensor(wl.gather_index[r], dtype=torch.long)].float() @ w1[int(e)].float().t()
+        assert_close(out0[torch.as_tensor(r).cuda()], ref, f"{name} layer0 expert {e}")
+    if name == "C2":
+        return
+    # layer1: grouped GEMM with the top-k weight in the epilogue, then the gather-reduce
+    act, w2 = wl.tensors["act"], wl.tensors["w2"]
+    z = capi.grouped_gemm(act.cuda(), w2.cuda(), split_d, row_scale=wl.row_weight.cuda())
+    for e in np.unique(eor[rows]):
+        r = rows[eor[rows] == e]
+        ref = (act[torch.as_tensor(r)].float() @ w2[int(e)].float().t()) * wl.row_weight[torch.as_tensor(r)][:, None]
+        assert_close(z[torch.as_tensor(r).cuda()], ref, f"{name} layer1 gemm expert {e}")
+    out1 = capi.topk_gather_reduce(z, torch.from_numpy(wl.scatter_index.reshape(-1)).cuda(), wl.topk)
+    tok = rng.integers(0, wl.tokens, size=48)
+    ref1 = torch.zeros(len(tok), wl.hidden)
+    for i, t in enumerate(tok):
+        for j in range(wl.topk):
+            r = int(wl.scatter_index[t, j])
+            ref1[i] += float(wl.row_weight[r]) * (act[r].float() @ w2[int(eor[r])].float().t())
+    assert_close(out1[torch.as_tensor(tok).cuda()], ref1, f"{name} layer1 output")
+
+
+def quantise(t_bf16):
+    bits = t_bf16.reshape(-1, t_bf16.shape[-1]).view(torch.int16).numpy().view(np.uint16)
+    q, s = quant.quant_rows_c(bits)
+    return torch.from_numpy(q).view(torch.float8_e4m3fn).reshape(t_bf16.shape), torch.from_numpy(s)
+
+
+@pytest.mark.parametrize("experts,rows,n,k,seed", [(1, 256, 256, 64, 0), (4, 1000, 512, 256, 1), (8, 2000, 1024, 1024, 2),
+                                                   (3, 300, 264, 2048, 3), (2, 40, 8, 100, 4)])
+def test_fp8_against_dequant_matmul(experts, rows, n, k, seed):
+    from flux_amd import capi
+    print(f"[case] grouped_gemm fp8 E={experts} rows={rows} N={n} K={k}", flush=True)
+    rng = np.random.default_rng(seed)
+    g = torch.Generator().manual_seed(seed)
+    split = random_splits(rng, experts, rows)
+    a = torch.randn(rows, k, generator=g).to(torch.bfloat16)
+    w = (torch.randn(experts, n, k, generator=g) * 0.02).to(torch.bfloat16)
+    qa, sa = quantise(a)
+    qw, sw = quantise(w)
+    sw = sw.reshape(experts, n)
+    tw = torch.rand(rows, generator=g) + 0.5
+    ref = layers.fp8_grouped_gemm_fp32(qa, sa, qw, sw, split, row_weight=tw)
+    out = capi.grouped_gemm(qa.cuda(), qw.cuda(), torch.from_numpy(split).cuda(), row_scale=(sa * tw).cuda(),
+                            col_scale=sw.cuda())
+    err = float((out.float().cpu() - ref).norm() / ref.norm())
+    assert err < FP8_FROB, err
+    assert err < 5e-3, err  # only accumulation order and the bf16 output rounding differ from the oracle
+
+
+def test_fp8_benchmark_c5_layer1():
+    """C5 at full size: quantise on the GPU, fp8 grouped GEMM with row x column scales and the top-8 weight in
+    the epilogue, gather-reduce; sampled rows / tokens against the dequantise-matmul oracle."""
+    from flux_amd import capi
+    wl = configs.make_workload("C5")
+    print(f"[case] grouped_gemm fp8 C5 M={wl.rows} K={wl.ffn} N={wl.hidden}", flush=True)
+    rng = np.random.default_rng(71)
+    act, w2 = wl.tensors["act"], wl.tensors["w2"]
+    qa_d, sa_d = capi.quant_e4m3(act.cuda())
+    qw_d, sw_d = capi.quant_e4m3(w2.reshape(-1, wl.ffn).cuda())
+    qw_d = qw_d.reshape(wl.experts, wl.hidden, wl.ffn)
+    sw_d = sw_d.reshape(wl.experts, wl.hidden)
+    split_d = torch.from_numpy(wl.splits).cuda()
+    z = capi.grouped_gemm(qa_d, qw_d, split_d, row_scale=sa_d * wl.row_weight.cuda(), col_scale=sw_d)
+    out = capi.topk_gather_reduce(z, torch.from_numpy(wl.scatter_index.reshape(-1)).cuda(), wl.topk)
+    eor = routing.expert_of_row(wl.splits)
+    rows = sampled_rows(wl.splits, 8, rng)
+    qa, sa, qw, sw = qa_d.cpu(), sa_d.cpu(), qw_d.cpu(), sw_d.cpu()
+    num = den = 0.0
+    for e in np.unique(eor[rows]):
+        r = torch.as_tensor(rows[eor[rows] == e])
+        ref = (qa[r].float() * sa[r][:, None]) @ (qw[int(e)].float() * sw[int(e)][:, None]).t() * wl.row_weight[r][:, None]
+        num += float((z[r.cuda()].float().cpu() - ref).pow(2).sum())
+        den += float(ref.pow(2).sum())
+    assert (num / den) ** 0.5 < FP8_FROB
+    tok = rng.integers(0, wl.tokens, size=16)
+    ref1 = torch.zeros(len(tok), wl.hidden)
+    for i, t in enumerate(tok):
+        for j in range(wl.topk):
+            r = int(wl.scatter_index[t, j])
+            e = int(eor[r])
+            ref1[i] += float(wl.row_weight[r]) * float(sa[r]) * ((qa[r].float() @ qw[e].float().t()) * sw[e])
+    got = out[torch.as_tensor(tok).cuda()].float().cpu()
+    assert float((got - ref1).norm() / ref1.norm()) < FP8_FROB
