@@ -30,7 +30,7 @@ class GroupedGemmArgs(ctypes.Structure):
         ("a", ctypes.c_void_p), ("b", ctypes.c_void_p), ("d", ctypes.c_void_p),
         ("splits", ctypes.c_void_p), ("gather_a", ctypes.c_void_p), ("scatter_d", ctypes.c_void_p),
         ("alpha", ctypes.c_void_p), ("row_scale", ctypes.c_void_p), ("col_scale", ctypes.c_void_p),
-        ("scalar_scale", ctypes.c_float), ("reserved1", ctypes.c_int32),
+        ("scalar_scale", ctypes.c_float), ("d_fp32", ctypes.c_int32),
         ("scalar_scale_dev", ctypes.c_void_p),
     ]
 
@@ -59,7 +59,7 @@ def load():
     lib.fluxmi_grouped_gemm_workspace_bytes.restype = sz
     lib.fluxmi_grouped_gemm_workspace_bytes.argtypes = [ctypes.POINTER(GroupedGemmArgs)]
     lib.fluxmi_grouped_gemm.argtypes = [ctypes.POINTER(GroupedGemmArgs), vp, sz, vp]
-    lib.fluxmi_topk_gather_reduce.argtypes = [ctypes.POINTER(vp), i32, vp, vp, f32, i32, i32, i32, vp, vp]
+    lib.fluxmi_topk_gather_reduce.argtypes = [ctypes.POINTER(vp), i32, i32, vp, vp, f32, i32, i32, i32, vp, vp]
     lib.fluxmi_quant_e4m3_rowwise.argtypes = [vp, i64, i64, i32, f32, vp, vp, i32, vp]
     _lib = lib
     return lib
@@ -117,7 +117,7 @@ def gather_index(scatter_index, topk):
 
 
 def grouped_gemm(a, b, splits, out=None, gather_a=None, scatter_d=None, alpha=None, row_scale=None,
-                 col_scale=None, scalar_scale=1.0, scalar_scale_dev=None, max_rows=None):
+                 col_scale=None, scalar_scale=1.0, scalar_scale_dev=None, max_rows=None, out_dtype=None):
     """D = grouped GEMM of A [rows_a, K] with B [E, N, K]; see fluxmi_grouped_gemm in include/fluxmi.h."""
     lib = load()
     if a.dtype == torch.bfloat16:
@@ -140,8 +140,10 @@ def grouped_gemm(a, b, splits, out=None, gather_a=None, scatter_d=None, alpha=No
     if max_rows is None:
         max_rows = gather_a.numel() if gather_a is not None else a.shape[0]
     if out is None:
-        out = torch.empty(max_rows, n, dtype=torch.bfloat16, device=a.device)
-    _dev_tensor(out, torch.bfloat16, "out")
+        out = torch.empty(max_rows, n, dtype=out_dtype or torch.bfloat16, device=a.device)
+    if out.dtype not in (torch.bfloat16, torch.float32):
+        raise ValueError(f"out must be bf16 or fp32, got {out.dtype}")
+    _dev_tensor(out, out.dtype, "out")
     if out.shape[0] < max_rows or out.shape[1] != n:
         raise ValueError(f"out {tuple(out.shape)} too small for [{max_rows}, {n}]")
     args = GroupedGemmArgs(
@@ -152,7 +154,7 @@ def grouped_gemm(a, b, splits, out=None, gather_a=None, scatter_d=None, alpha=No
         alpha=None if alpha is None else alpha.data_ptr(),
         row_scale=None if row_scale is None else row_scale.data_ptr(),
         col_scale=None if col_scale is None else col_scale.data_ptr(),
-        scalar_scale=float(scalar_scale), reserved1=0,
+        scalar_scale=float(scalar_scale), d_fp32=int(out.dtype == torch.float32),
         scalar_scale_dev=None if scalar_scale_dev is None else scalar_scale_dev.data_ptr())
     _check(lib.fluxmi_grouped_gemm(ctypes.byref(args), None, 0, _stream()), "fluxmi_grouped_gemm")
     return out
@@ -163,8 +165,11 @@ def topk_gather_reduce(inputs, routing_idx, topk, row_weight=None, scale=1.0, ou
     lib = load()
     if isinstance(inputs, torch.Tensor):
         inputs = [inputs]
+    in_dtype = inputs[0].dtype
+    if in_dtype not in (torch.bfloat16, torch.float32):
+        raise ValueError(f"inputs must be bf16 or fp32, got {in_dtype}")
     for g, t in enumerate(inputs):
-        _dev_tensor(t, torch.bfloat16, f"inputs[{g}]")
+        _dev_tensor(t, in_dtype, f"inputs[{g}]")
     _dev_tensor(routing_idx, torch.int32, "routing_idx")
     _dev_tensor(row_weight, torch.float32, "row_weight")
     m, n = inputs[0].shape
@@ -174,7 +179,7 @@ def topk_gather_reduce(inputs, routing_idx, topk, row_weight=None, scale=1.0, ou
     if out is None:
         out = torch.empty(ntokens, n, dtype=torch.bfloat16, device=inputs[0].device)
     ptrs = (ctypes.c_void_p * len(inputs))(*[t.data_ptr() for t in inputs])
-    _check(lib.fluxmi_topk_gather_reduce(ptrs, len(inputs), _ptr(routing_idx), _ptr(row_weight),
+    _check(lib.fluxmi_topk_gather_reduce(ptrs, len(inputs), int(in_dtype == torch.float32), _ptr(routing_idx), _ptr(row_weight),
                                          float(scale), ntokens, topk, n, _ptr(out), _stream()),
            "fluxmi_topk_gather_reduce")
     return out

@@ -13,12 +13,45 @@ constexpr int kMaxGroups = 4;
 constexpr int kThreads = 256;
 
 struct GroupPtrs {
-  const uint16_t *p[kMaxGroups];
+  const void *p[kMaxGroups];
 };
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-__device__ __forceinline__ void accumulate8(float (&acc)[8], const u32x4 v, const float w) {
+// Eight consecutive elements of a source row as loaded: one 16-byte vector of bf16, or two of fp32.
+template <bool IN_F32>
+struct Vec8 {
+  u32x4 v[IN_F32 ? 2 : 1];
+};
+
+template <bool IN_F32>
+__device__ __forceinline__ Vec8<IN_F32> load8(const void *base, size_t row, size_t row_vecs, int v) {
+  Vec8<IN_F32> r;
+  if constexpr (IN_F32) {
+    const u32x4 *src = reinterpret_cast<const u32x4 *>(base) + (row * row_vecs + v) * 2;
+    r.v[0] = __builtin_nontemporal_load(src);
+    r.v[1] = __builtin_nontemporal_load(src + 1);
+  } else {
+    r.v[0] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(base) + row * row_vecs + v);
+  }
+  return r;
+}
+
+template <bool IN_F32>
+__device__ __forceinline__ Vec8<IN_F32> zero8() {
+  Vec8<IN_F32> r;
+#pragma unroll
+  for (int i = 0; i < (IN_F32 ? 2 : 1); ++i) r.v[i] = u32x4{0u, 0u, 0u, 0u};
+  return r;
+}
+
+__device__ __forceinline__ void accumulate8(float (&acc)[8], const Vec8<true> &x, const float w) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i) acc[i] = fmaf(w, __uint_as_float(x.v[i >> 2][i & 3]), acc[i]);
+}
+
+__device__ __forceinline__ void accumulate8(float (&acc)[8], const Vec8<false> &x, const float w) {
+  const u32x4 v = x.v[0];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const uint32_t u = v[i];
@@ -28,7 +61,7 @@ __device__ __forceinline__ void accumulate8(float (&acc)[8], const u32x4 v, cons
 }
 
 // TOPK > 0: compile-time top-k (loads fully unrolled).  TOPK == 0: run-time top-k.
-template <int TOPK, int NGROUPS, bool WEIGHTED>
+template <int TOPK, int NGROUPS, bool WEIGHTED, bool IN_F32>
 __global__ __launch_bounds__(kThreads) void topk_gather_reduce_kernel(
     GroupPtrs in, const int32_t *__restrict__ routing_idx, const float *__restrict__ row_weight,
     float scale, int32_t topk_rt, int32_t nvec /* n / 8 */, uint16_t *__restrict__ out) {
@@ -39,7 +72,7 @@ __global__ __launch_bounds__(kThreads) void topk_gather_reduce_kernel(
   for (int v = blockIdx.y * kThreads + threadIdx.x; v < nvec; v += gridDim.y * kThreads) {
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     if constexpr (TOPK > 0) {
-      u32x4 vals[NGROUPS][TOPK];
+      Vec8<IN_F32> vals[NGROUPS][TOPK];
       float w[TOPK];
 #pragma unroll
       for (int j = 0; j < TOPK; ++j) {
@@ -48,12 +81,9 @@ __global__ __launch_bounds__(kThreads) void topk_gather_reduce_kernel(
         if (r >= 0) w[j] = WEIGHTED ? row_weight[r] : 1.f;
 #pragma unroll
         for (int g = 0; g < NGROUPS; ++g) {
-          vals[g][j] = u32x4{0u, 0u, 0u, 0u};
-          if (r >= 0) {  // r is wave-uniform: a skipped (dropped) row costs no traffic
-            const u32x4 *src =
-                reinterpret_cast<const u32x4 *>(in.p[g]) + static_cast<size_t>(r) * row_vecs + v;
-            vals[g][j] = __builtin_nontemporal_load(src);
-          }
+          vals[g][j] = zero8<IN_F32>();
+          // r is wave-uniform: a skipped (dropped) row costs no traffic
+          if (r >= 0) vals[g][j] = load8<IN_F32>(in.p[g], static_cast<size_t>(r), row_vecs, v);
         }
       }
 #pragma unroll
@@ -67,9 +97,7 @@ __global__ __launch_bounds__(kThreads) void topk_gather_reduce_kernel(
           const int32_t r = routing_idx[static_cast<size_t>(t) * topk + j];
           if (r < 0) continue;
           const float w = WEIGHTED ? row_weight[r] : 1.f;
-          const u32x4 *src =
-              reinterpret_cast<const u32x4 *>(in.p[g]) + static_cast<size_t>(r) * row_vecs + v;
-          accumulate8(acc, __builtin_nontemporal_load(src), w);
+          accumulate8(acc, load8<IN_F32>(in.p[g], static_cast<size_t>(r), row_vecs, v), w);
         }
       }
     }
@@ -86,33 +114,38 @@ __global__ __launch_bounds__(kThreads) void topk_gather_reduce_kernel(
 }
 
 template <int TOPK, int NGROUPS>
-void launch(bool weighted, dim3 grid, hipStream_t s, const GroupPtrs &in, const int32_t *idx,
-            const float *w, float scale, int32_t topk, int32_t nvec, uint16_t *out) {
-  if (weighted)
-    hipLaunchKernelGGL((topk_gather_reduce_kernel<TOPK, NGROUPS, true>), grid, dim3(kThreads), 0, s,
-                       in, idx, w, scale, topk, nvec, out);
-  else
-    hipLaunchKernelGGL((topk_gather_reduce_kernel<TOPK, NGROUPS, false>), grid, dim3(kThreads), 0, s,
-                       in, idx, w, scale, topk, nvec, out);
+void launch(bool weighted, bool in_f32, dim3 grid, hipStream_t s, const GroupPtrs &in,
+            const int32_t *idx, const float *w, float scale, int32_t topk, int32_t nvec, uint16_t *out) {
+#define FLUXMI_GR_LAUNCH(W, F)                                                                        \
+  hipLaunchKernelGGL((topk_gather_reduce_kernel<TOPK, NGROUPS, W, F>), grid, dim3(kThreads), 0, s, in, \
+                     idx, w, scale, topk, nvec, out)
+  if (weighted) {
+    if (in_f32) FLUXMI_GR_LAUNCH(true, true);
+    else FLUXMI_GR_LAUNCH(true, false);
+  } else {
+    if (in_f32) FLUXMI_GR_LAUNCH(false, true);
+    else FLUXMI_GR_LAUNCH(false, false);
+  }
+#undef FLUXMI_GR_LAUNCH
 }
 
 template <int NGROUPS>
-void dispatch_topk(bool weighted, dim3 grid, hipStream_t s, const GroupPtrs &in, const int32_t *idx,
+void dispatch_topk(bool weighted, bool in_f32, dim3 grid, hipStream_t s, const GroupPtrs &in, const int32_t *idx,
                    const float *w, float scale, int32_t topk, int32_t nvec, uint16_t *out) {
   switch (topk) {
-    case 1: launch<1, NGROUPS>(weighted, grid, s, in, idx, w, scale, topk, nvec, out); break;
-    case 2: launch<2, NGROUPS>(weighted, grid, s, in, idx, w, scale, topk, nvec, out); break;
-    case 4: launch<4, NGROUPS>(weighted, grid, s, in, idx, w, scale, topk, nvec, out); break;
-    case 6: launch<6, NGROUPS>(weighted, grid, s, in, idx, w, scale, topk, nvec, out); break;
-    case 8: launch<8, NGROUPS>(weighted, grid, s, in, idx, w, scale, topk, nvec, out); break;
-    default: launch<0, NGROUPS>(weighted, grid, s, in, idx, w, scale, topk, nvec, out); break;
+    case 1: launch<1, NGROUPS>(weighted, in_f32, grid, s, in, idx, w, scale, topk, nvec, out); break;
+    case 2: launch<2, NGROUPS>(weighted, in_f32, grid, s, in, idx, w, scale, topk, nvec, out); break;
+    case 4: launch<4, NGROUPS>(weighted, in_f32, grid, s, in, idx, w, scale, topk, nvec, out); break;
+    case 6: launch<6, NGROUPS>(weighted, in_f32, grid, s, in, idx, w, scale, topk, nvec, out); break;
+    case 8: launch<8, NGROUPS>(weighted, in_f32, grid, s, in, idx, w, scale, topk, nvec, out); break;
+    default: launch<0, NGROUPS>(weighted, in_f32, grid, s, in, idx, w, scale, topk, nvec, out); break;
   }
 }
 
 }  // namespace
 }  // namespace fluxmi
 
-extern "C" int fluxmi_topk_gather_reduce(const void *const *in, int32_t ngroups,
+extern "C" int fluxmi_topk_gather_reduce(const void *const *in, int32_t ngroups, int32_t in_fp32,
                                          const int32_t *routing_idx, const float *row_weight,
                                          float scale, int32_t ntokens, int32_t topk, int32_t n,
                                          void *out, void *stream) {
@@ -131,7 +164,7 @@ extern "C" int fluxmi_topk_gather_reduce(const void *const *in, int32_t ngroups,
   for (int g = 0; g < ngroups; ++g) {
     FLUXMI_REQUIRE(in[g] != nullptr && aligned16(in[g]), FLUXMI_ERR_INVALID_ARG,
                    "topk_gather_reduce: input group %d is null or not 16-byte aligned", g);
-    gp.p[g] = static_cast<const uint16_t *>(in[g]);
+    gp.p[g] = in[g];
   }
   FLUXMI_REQUIRE(aligned16(out), FLUXMI_ERR_INVALID_ARG,
                  "topk_gather_reduce: output is not 16-byte aligned");
@@ -150,10 +183,10 @@ extern "C" int fluxmi_topk_gather_reduce(const void *const *in, int32_t ngroups,
   const bool weighted = row_weight != nullptr;
   uint16_t *o = static_cast<uint16_t *>(out);
   switch (ngroups) {
-    case 1: dispatch_topk<1>(weighted, grid, s, gp, routing_idx, row_weight, scale, topk, nvec, o); break;
-    case 2: dispatch_topk<2>(weighted, grid, s, gp, routing_idx, row_weight, scale, topk, nvec, o); break;
-    case 3: dispatch_topk<3>(weighted, grid, s, gp, routing_idx, row_weight, scale, topk, nvec, o); break;
-    default: dispatch_topk<4>(weighted, grid, s, gp, routing_idx, row_weight, scale, topk, nvec, o); break;
+    case 1: dispatch_topk<1>(weighted, in_fp32 != 0, grid, s, gp, routing_idx, row_weight, scale, topk, nvec, o); break;
+    case 2: dispatch_topk<2>(weighted, in_fp32 != 0, grid, s, gp, routing_idx, row_weight, scale, topk, nvec, o); break;
+    case 3: dispatch_topk<3>(weighted, in_fp32 != 0, grid, s, gp, routing_idx, row_weight, scale, topk, nvec, o); break;
+    default: dispatch_topk<4>(weighted, in_fp32 != 0, grid, s, gp, routing_idx, row_weight, scale, topk, nvec, o); break;
   }
   FLUXMI_HIP_CHECK(hipGetLastError());
   return FLUXMI_OK;

@@ -42,7 +42,7 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 struct GemmParams {
   const uint8_t *a;
   const uint8_t *b;
-  uint16_t *d;
+  void *d;
   const int32_t *splits;
   const int32_t *gather_a;
   const int32_t *scatter_d;
@@ -56,6 +56,7 @@ struct GemmParams {
   int32_t a_rows;
   int32_t n;
   int32_t k;
+  int32_t d_fp32;
 };
 
 #define FLUXMI_WAITCNT(vm, lgkm) \
@@ -284,7 +285,8 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
         drow = p.scatter_d[srow];
         if (drow < 0 || drow >= p.max_rows) continue;
       }
-      uint16_t *dptr = p.d + drow * p.n;
+      uint16_t *dptr = static_cast<uint16_t *>(p.d) + drow * p.n;
+      float *dptr32 = static_cast<float *>(p.d) + drow * p.n;
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
 #pragma unroll
@@ -303,10 +305,14 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
             v2 *= cs.z;
             v3 *= cs.w;
           }
-          u32x2 o;
-          o[0] = float_to_bf16_bits(v0) | (static_cast<uint32_t>(float_to_bf16_bits(v1)) << 16);
-          o[1] = float_to_bf16_bits(v2) | (static_cast<uint32_t>(float_to_bf16_bits(v3)) << 16);
-          *reinterpret_cast<u32x2 *>(dptr + n) = o;
+          if (p.d_fp32) {
+            *reinterpret_cast<float4 *>(dptr32 + n) = make_float4(v0, v1, v2, v3);
+          } else {
+            u32x2 o;
+            o[0] = float_to_bf16_bits(v0) | (static_cast<uint32_t>(float_to_bf16_bits(v1)) << 16);
+            o[1] = float_to_bf16_bits(v2) | (static_cast<uint32_t>(float_to_bf16_bits(v3)) << 16);
+            *reinterpret_cast<u32x2 *>(dptr + n) = o;
+          }
         }
       }
     }
@@ -374,7 +380,8 @@ __global__ __launch_bounds__(256) void grouped_gemm_generic_kernel(const GemmPar
       drow = p.scatter_d[r];
       if (drow < 0 || drow >= p.max_rows) continue;
     }
-    p.d[drow * p.n + n] = float_to_bf16_bits(v);
+    if (p.d_fp32) static_cast<float *>(p.d)[drow * p.n + n] = v;
+    else static_cast<uint16_t *>(p.d)[drow * p.n + n] = float_to_bf16_bits(v);
   }
 }
 
@@ -382,7 +389,7 @@ bool mfma_path_ok(const fluxmi_grouped_gemm_args *a) {
   const int elt = a->dtype == FLUXMI_BF16 ? 2 : 1;
   const int64_t kbytes = static_cast<int64_t>(a->k) * elt;
   return kbytes % KBYTES == 0 && kbytes >= KBYTES && a->n % 4 == 0 && aligned16(a->a) &&
-         aligned16(a->b) && (reinterpret_cast<uintptr_t>(a->d) & 7u) == 0 &&
+         aligned16(a->b) && (reinterpret_cast<uintptr_t>(a->d) & (a->d_fp32 ? 15u : 7u)) == 0 &&
          (a->col_scale == nullptr || aligned16(a->col_scale));
 }
 
@@ -400,7 +407,8 @@ extern "C" int fluxmi_grouped_gemm(const fluxmi_grouped_gemm_args *args, void *,
   FLUXMI_REQUIRE(args != nullptr, FLUXMI_ERR_INVALID_ARG, "grouped_gemm: null args");
   FLUXMI_REQUIRE(args->dtype == FLUXMI_BF16 || args->dtype == FLUXMI_FP8_E4M3, FLUXMI_ERR_INVALID_ARG,
                  "grouped_gemm: unknown dtype %d", args->dtype);
-  FLUXMI_REQUIRE(args->reserved1 == 0, FLUXMI_ERR_INVALID_ARG, "grouped_gemm: reserved field must be 0");
+  FLUXMI_REQUIRE(args->d_fp32 == 0 || args->d_fp32 == 1, FLUXMI_ERR_INVALID_ARG,
+                 "grouped_gemm: d_fp32 must be 0 or 1");
   FLUXMI_REQUIRE(args->a_rows >= 0, FLUXMI_ERR_INVALID_ARG, "grouped_gemm: negative a_rows");
   FLUXMI_REQUIRE(args->nexperts >= 1 && args->nexperts <= kMaxExperts, FLUXMI_ERR_UNSUPPORTED,
                  "grouped_gemm: nexperts=%d outside [1,%d]", args->nexperts, kMaxExperts);
@@ -415,7 +423,7 @@ extern "C" int fluxmi_grouped_gemm(const fluxmi_grouped_gemm_args *args, void *,
   GemmParams p;
   p.a = static_cast<const uint8_t *>(args->a);
   p.b = static_cast<const uint8_t *>(args->b);
-  p.d = static_cast<uint16_t *>(args->d);
+  p.d = args->d;
   p.splits = args->splits;
   p.gather_a = args->gather_a;
   p.scatter_d = args->scatter_d;
@@ -429,6 +437,7 @@ extern "C" int fluxmi_grouped_gemm(const fluxmi_grouped_gemm_args *args, void *,
   p.a_rows = args->a_rows;
   p.n = args->n;
   p.k = args->k;
+  p.d_fp32 = args->d_fp32;
 
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int cus = fluxmi_device_cu_count();

@@ -175,7 +175,7 @@ extern "C" int fluxmi_moe_route_sort(const int32_t *choosed, int32_t ntokens, in
   const int64_t npairs64 = static_cast<int64_t>(ntokens) * topk;
   FLUXMI_REQUIRE(npairs64 <= (int64_t{1} << 30), FLUXMI_ERR_UNSUPPORTED,
                  "moe_route_sort: ntokens*topk=%lld exceeds 2^30", static_cast<long long>(npairs64));
-  FLUXMI_REQUIRE(scatter_index != nullptr && (choosed != nullptr || npairs64 == 0),
+  FLUXMI_REQUIRE((scatter_index != nullptr && choosed != nullptr) || npairs64 == 0,
                  FLUXMI_ERR_INVALID_ARG, "moe_route_sort: null choosed / scatter_index");
   const size_t need = fluxmi_moe_route_sort_workspace_bytes(ntokens, topk, nexperts);
   FLUXMI_REQUIRE(workspace != nullptr && workspace_bytes >= need, FLUXMI_ERR_WORKSPACE,

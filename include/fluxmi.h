@@ -96,7 +96,7 @@ typedef struct fluxmi_grouped_gemm_args {
   int32_t a_rows;        /* rows of A when gather_a is given: entries are clamped into [0, a_rows); 0 = trust them */
   const void *a;         /* [rows_a, K] */
   const void *b;         /* [E, N, K] */
-  void *d;               /* [max_rows, N] bf16 */
+  void *d;               /* [max_rows, N] bf16 (fp32 when d_fp32 != 0) */
   const int32_t *splits; /* device [E] */
   const int32_t *gather_a;  /* device [max_rows] or NULL */
   const int32_t *scatter_d; /* device [max_rows] or NULL */
@@ -104,7 +104,7 @@ typedef struct fluxmi_grouped_gemm_args {
   const float *row_scale;   /* device [max_rows] or NULL, indexed by sorted row */
   const float *col_scale;   /* device [E, N] or NULL */
   float scalar_scale;       /* host scalar, 1.0f for none (Flux `input_scale[0]` is passed by pointer below) */
-  int32_t reserved1;        /* must be 0 */
+  int32_t d_fp32;           /* 0: D is bf16; 1: D is fp32 [max_rows, N] (unrounded layer1 intermediate) */
   const float *scalar_scale_dev; /* device [1] or NULL; multiplied in if given */
 } fluxmi_grouped_gemm_args;
 
@@ -124,12 +124,13 @@ int fluxmi_grouped_gemm(const fluxmi_grouped_gemm_args *args, void *workspace,
  *                       w[r] * float(in[g][r, n]) ),   r = routing_idx[t*topk + j],
  *   w[r] = row_weight ? row_weight[r] : 1;  rows with r < 0 are skipped; fp32 accumulation in the
  *   order g-major then j; one rounding at the end.
- * `in` is an array (on the HOST) of `ngroups` device pointers to row-major bf16 [nrows, n] matrices.
+ * `in` is an array (on the HOST) of `ngroups` device pointers to row-major [nrows, n] matrices, bf16, or
+ * fp32 when `in_fp32` != 0 (the unrounded intermediate of fluxmi_grouped_gemm with d_fp32 = 1).
  * Requirements: n % 8 == 0, 1 <= ngroups <= 4, 1 <= topk <= 64.
  * ---------------------------------------------------------------------------------------------- */
-int fluxmi_topk_gather_reduce(const void *const *in, int32_t ngroups, const int32_t *routing_idx,
-                              const float *row_weight, float scale, int32_t ntokens, int32_t topk,
-                              int32_t n, void *out, void *stream);
+int fluxmi_topk_gather_reduce(const void *const *in, int32_t ngroups, int32_t in_fp32,
+                              const int32_t *routing_idx, const float *row_weight, float scale,
+                              int32_t ntokens, int32_t topk, int32_t n, void *out, void *stream);
 
 /* ------------------------------------------------------------------------------------------------
  * bf16 -> fp8-e4m3 absmax quantisation, one scale per (row, block of `block_cols` columns).

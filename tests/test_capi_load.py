@@ -31,12 +31,12 @@ def test_argument_errors_without_gpu():
     """Validation happens before any HIP call, so it is testable on a CPU-only host."""
     from flux_amd import capi
     lib = capi.load()
-    rc = lib.fluxmi_topk_gather_reduce(None, 1, None, None, 1.0, 4, 2, 64, None, None)
+    rc = lib.fluxmi_topk_gather_reduce(None, 1, 0, None, None, 1.0, 4, 2, 64, None, None)
     assert rc == -1 and b"null pointer" in lib.fluxmi_last_error()
     ptrs = (ctypes.c_void_p * 1)(0x1000)
-    rc = lib.fluxmi_topk_gather_reduce(ptrs, 9, ctypes.c_void_p(0x1000), None, 1.0, 4, 2, 64, ctypes.c_void_p(0x1000), None)
+    rc = lib.fluxmi_topk_gather_reduce(ptrs, 9, 0, ctypes.c_void_p(0x1000), None, 1.0, 4, 2, 64, ctypes.c_void_p(0x1000), None)
     assert rc == -2 and b"ngroups" in lib.fluxmi_last_error()
-    rc = lib.fluxmi_topk_gather_reduce(ptrs, 1, ctypes.c_void_p(0x1000), None, 1.0, 4, 2, 60, ctypes.c_void_p(0x1000), None)
+    rc = lib.fluxmi_topk_gather_reduce(ptrs, 1, 0, ctypes.c_void_p(0x1000), None, 1.0, 4, 2, 60, ctypes.c_void_p(0x1000), None)
     assert rc == -2 and b"multiple of 8" in lib.fluxmi_last_error()
     rc = lib.fluxmi_quant_e4m3_rowwise(ctypes.c_void_p(0x1000), 4, 64, 32, 0.0, ctypes.c_void_p(0x1000),
                                        ctypes.c_void_p(0x1000), 0, None)

@@ -35,6 +35,19 @@ def test_against_oracle(tokens, topk, n, weighted, groups, seed):
     assert_close(out, ref)
 
 
+@pytest.mark.parametrize("tokens,topk,n,groups", [(64, 2, 1024, 1), (100, 6, 1408, 1), (9, 3, 264, 2), (300, 7, 512, 1)])
+def test_fp32_intermediate_input(tokens, topk, n, groups):
+    from flux_amd import capi
+    g = torch.Generator().manual_seed(tokens)
+    m = tokens * topk
+    inter = [torch.randn(m, n, generator=g) for _ in range(groups)]
+    idx = torch.randperm(m, generator=g).to(torch.int32)
+    w = torch.rand(m, generator=g)
+    ref = layers.topk_gather_reduce_fp32(inter, idx.numpy(), topk, w, scale=2.0)
+    out = capi.topk_gather_reduce([t.cuda() for t in inter], idx.cuda(), topk, w.cuda(), 2.0)
+    assert_close(out, ref)
+
+
 def test_dropped_rows_and_identity():
     from flux_amd import capi
     g = torch.Generator().manual_seed(9)

@@ -97,5 +97,6 @@ def test_benchmark_shapes(rows, cols):
     deq = q.float() * s[:, None]
     amax = x.float().abs().amax(1)
     assert bool((q.float().abs().amax(1) == 448.0).all())
-    assert bool(((deq - x.float()).abs() <= amax[:, None] / 448.0 * 16.0).all())
+    # half of the widest e4m3 step (32, between 256 and 448), in input units; ties reach it exactly, hence the slack
+    assert bool(((deq - x.float()).abs() <= amax[:, None] / 448.0 * 16.0 * 1.001).all())
     assert torch.allclose(s * (448.0 / amax), torch.ones_like(s), rtol=1e-6)
