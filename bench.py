@@ -1,0 +1,208 @@
+"""Benchmark of the MoE hot path on one MI355X.
+
+A step = one pass of the path over one batch: routing sort -> layer0 (row gather fused into the grouped
+GEMM) -> layer1 grouped GEMM (top-k weight in the epilogue) -> top-k gather-reduce to token order.
+Workload at N=1: C3, the Mixtral-shape layer the metric is quoted on (T=8192, H=4096, F=14336, E=8,
+top-2, bf16), synthetic data, inputs resident in HBM before the timed region.
+
+Prints ONE JSON line: whole-step throughput in TFLOP/s (algorithmic GEMM FLOPs of the step / step
+time), the roofline object of the dominant kernel (grouped GEMM, MFMA-bound) measured with HIP events
+inside the timed region, per-kernel figures, and the CPU oracle timed on a bounded sample.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+METRIC = "grouped-GEMM TFLOP/s (% MFMA peak) + gather-reduce GB/s, Mixtral shape, 1 GPU"
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
+PEAK_FP8_TFLOPS = 5000.0
+PEAK_HBM_GBS = 8000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="C3", choices=["C1", "C3", "C4"])
+    ap.add_argument("--inter", default="fp32", choices=["fp32", "bf16"],
+                    help="dtype of the layer1 intermediate [M, H]")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-aux", action="store_true", help="skip the stand-alone HBM kernel measurements")
+    return ap.parse_args()
+
+
+class Events:
+    """HIP events (torch.cuda.Event on the stream the kernels are launched on) around named spans."""
+
+    def __init__(self, torch):
+        self.torch = torch
+        self.spans = {}
+
+    def span(self, name, fn):
+        e0 = self.torch.cuda.Event(enable_timing=True)
+        e1 = self.torch.cuda.Event(enable_timing=True)
+        e0.record()
+        out = fn()
+        e1.record()
+        self.spans.setdefault(name, []).append((e0, e1))
+        return out
+
+    def mean_ms(self, name):
+        v = [a.elapsed_time(b) for a, b in self.spans[name]]
+        return sum(v) / len(v)
+
+
+def time_loop(torch, fn, iters, warm=3):
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / iters
+
+
+def cpu_baseline(torch, wl_name, x, w1, w2):
+    """The CPU oracle (PyTorch-CPU restatement of the reference's torch layer) on a bounded sample:
+    the first 2048 tokens of the same workload, full hidden / ffn sizes."""
+    from oracle import configs, layers
+
+    sample_tokens = 2048 if wl_name != "C1" else 256
+    wl, _ = configs.make_routing(wl_name, tokens=sample_tokens)
+    threads = torch.get_num_threads()
+    xs = x[:sample_tokens].cpu()
+    w1c, w2c = w1.cpu(), w2.cpu()
+    t0 = time.perf_counter()
+    y = layers.layer0_fp32(xs, w1c, wl.splits, wl.gather_index).to(torch.bfloat16)
+    out = layers.layer1_fp32(y, w2c, wl.splits, wl.scatter_index.reshape(-1), wl.topk,
+                             output_vec_scale=wl.row_weight)
+    dt = time.perf_counter() - t0
+    flops = 2.0 * wl.rows * wl.hidden * wl.ffn * 2
+    assert out.shape == (sample_tokens, wl.hidden)
+    return {"value": round(flops / dt * 1e-12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": f"first {sample_tokens} tokens of {wl_name} (M={wl.rows} rows, full H/F), layer0+layer1, "
+                      f"fp32 matmul on bf16-valued inputs, {dt:.2f} s wall"}
+
+
+def main():
+    a = parse()
+    if a.gpus != 1:
+        print(f"bench.py measures one GPU only (got --gpus {a.gpus}): this build has no multi-GPU path",
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    from flux_amd import capi
+    from oracle import configs
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    dev = torch.device("cuda:0")
+    capi.load()
+
+    wl, _ = configs.make_routing(a.workload)
+    t, k, e, h, f, m = wl.tokens, wl.topk, wl.experts, wl.hidden, wl.ffn, wl.rows
+    gen = torch.Generator(device=dev).manual_seed(1000)
+    x = torch.randn(t, h, generator=gen, device=dev).to(torch.bfloat16)
+    w1 = (torch.randn(e, f, h, generator=gen, device=dev) * 0.02).to(torch.bfloat16)
+    w2 = (torch.randn(e, h, f, generator=gen, device=dev) * 0.02).to(torch.bfloat16)
+    choosed = wl.choosed.to(dev)
+    row_w = wl.row_weight.to(dev)
+    inter_dtype = torch.float32 if a.inter == "fp32" else torch.bfloat16
+    y = torch.empty(m, f, dtype=torch.bfloat16, device=dev)
+    z = torch.empty(m, h, dtype=inter_dtype, device=dev)
+    out = torch.empty(t, h, dtype=torch.bfloat16, device=dev)
+
+    ev = Events(torch)
+
+    def step(rec):
+        span = rec.span if rec else (lambda _n, fn: fn())
+        splits, _off, scatter, gather, _tki = span("route_sort", lambda: capi.route_sort(choosed, e))
+        span("gemm_layer0", lambda: capi.grouped_gemm(x, w1, splits, out=y, gather_a=gather))
+        span("gemm_layer1", lambda: capi.grouped_gemm(y, w2, splits, out=z, row_scale=row_w))
+        span("gather_reduce", lambda: capi.topk_gather_reduce(z, scatter.reshape(-1), k, out=out))
+
+    for _ in range(a.warmup):
+        step(None)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        step(ev)
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / a.steps
+
+    gemm_flops = 2.0 * m * h * f                      # per layer, actual routed rows only
+    step_flops = 2 * gemm_flops
+    ms = {n: ev.mean_ms(n) for n in ("route_sort", "gemm_layer0", "gemm_layer1", "gather_reduce")}
+    gemm_ms = 0.5 * (ms["gemm_layer0"] + ms["gemm_layer1"])
+    achieved = gemm_flops / gemm_ms * 1e-9            # TFLOP/s
+    inter_b = 4 if a.inter == "fp32" else 2
+    gr_bytes = m * h * inter_b + m * 4 + t * h * 2
+    route_bytes = m * 4 * 2 + e * 4 + 3 * m * 4       # pairs read twice, three index arrays written
+
+    kernels = {
+        "gemm_layer0": {"ms": round(ms["gemm_layer0"], 4), "tflops": round(gemm_flops / ms["gemm_layer0"] * 1e-9, 1)},
+        "gemm_layer1": {"ms": round(ms["gemm_layer1"], 4), "tflops": round(gemm_flops / ms["gemm_layer1"] * 1e-9, 1)},
+        "gather_reduce": {"ms": round(ms["gather_reduce"], 4), "gbs": round(gr_bytes / ms["gather_reduce"] * 1e-6, 1),
+                          "frac_hbm": round(gr_bytes / ms["gather_reduce"] * 1e-6 / PEAK_HBM_GBS, 4),
+                          "input": a.inter},
+        "route_sort": {"ms": round(ms["route_sort"], 4), "gbs": round(route_bytes / ms["route_sort"] * 1e-6, 1)},
+    }
+
+    if not a.no_aux:
+        # Stand-alone HBM kernels of the path that the step above does not exercise in this form.
+        zb = torch.randn(m, h, generator=gen, device=dev).to(torch.bfloat16)
+        sc = torch.from_numpy(wl.scatter_index.reshape(-1)).to(dev)
+        t_gr = time_loop(torch, lambda: capi.topk_gather_reduce(zb, sc, k, row_w, out=out), 50)
+        b_gr = m * h * 2 + m * 4 + m * 4 + t * h * 2
+        kernels["gather_reduce_bf16_weighted"] = {"ms": round(t_gr, 4), "gbs": round(b_gr / t_gr * 1e-6, 1),
+                                                  "frac_hbm": round(b_gr / t_gr * 1e-6 / PEAK_HBM_GBS, 4)}
+        for rows, cols in ((4096, 7168), (32768, 2048)):
+            xq = torch.randn(rows, cols, generator=gen, device=dev).to(torch.bfloat16)
+            t_q = time_loop(torch, lambda: capi.quant_e4m3(xq), 50)
+            b_q = rows * cols * 3 + rows * 4
+            kernels[f"quant_e4m3_{rows}x{cols}"] = {"ms": round(t_q, 4), "gbs": round(b_q / t_q * 1e-6, 1),
+                                                    "frac_hbm": round(b_q / t_q * 1e-6 / PEAK_HBM_GBS, 4)}
+        del zb
+
+    result = {
+        "metric": METRIC,
+        "value": round(step_flops / ms_per_step * 1e-9, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": a.steps,
+        "warmup": a.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"{a.workload}: tokens={t} topk={k} experts={e} hidden={h} ffn={f} rows={m}; "
+                               f"step = route sort + layer0 gather-GEMM + layer1 GEMM + top-k gather-reduce",
+                   "layer1_intermediate": a.inter,
+                   "rows_per_expert_min_max": [int(wl.splits.min()), int(wl.splits.max())]},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "kernel": "grouped_gemm_mfma_kernel<bf16>", "flop_per_launch": gemm_flops,
+                     "avg_launch_ms": round(gemm_ms, 4)},
+        "kernels": kernels,
+    }
+    if not a.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(torch, a.workload, x, w1, w2)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
