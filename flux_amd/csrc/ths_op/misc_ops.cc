@@ -1,0 +1,141 @@
+// Quantization (src/quantization/ths_op/quantization.{h,cc}) and the free functions of the reference's
+// module on this path: calc_scatter_index (src/pybind/ths_op.cc:59-78), topk_scatter_reduce
+// (src/moe_gather_rs/ths_op/topk_scatter_reduce.cc:30-56), bitwise_check (src/ths_op/ths_op.cc).
+#include "ths_ops.h"
+
+namespace flux_amd {
+
+constexpr int64_t kBlock = 128;  // BLOCK_TILE_DIM of the reference's quantisation kernels
+
+Quantization::Quantization(at::ScalarType input_dtype, at::ScalarType output_dtype, int32_t /*num_streams*/)
+    : input_dtype_(input_dtype), output_dtype_(output_dtype) {
+  // The reference hard-wires the same pair (src/quantization/quantization.cu:1399-1400).
+  TORCH_CHECK(input_dtype == at::kBFloat16, "Quantization: input dtype must be bfloat16, got ", input_dtype);
+  TORCH_CHECK(output_dtype == at::ScalarType::Float8_e4m3fn, "Quantization: output dtype must be float8_e4m3fn, got ",
+              output_dtype);
+}
+
+static void quant_call(const torch::Tensor &x, int32_t block_cols, float eps, torch::Tensor &q,
+                       torch::Tensor &scale_inv, bool permute) {
+  check_status(fluxmi_quant_e4m3_rowwise(x.data_ptr(), x.size(0), x.size(1), block_cols, eps, q.data_ptr(),
+                                         scale_inv.data_ptr<float>(), permute ? 1 : 0, current_stream()),
+               "fluxmi_quant_e4m3_rowwise");
+}
+
+Quantization::Result Quantization::quantize_vector_blockwise(torch::Tensor input, bool return_transpose, float eps) {
+  TORCH_CHECK(input.dim() == 2, "Input must have 2 dimensions.");
+  FLUX_AMD_CHECK_INPUT(input, input_dtype_);
+  const int64_t rows = input.size(0), cols = input.size(1);
+  const int64_t bx = (cols + kBlock - 1) / kBlock, by = (rows + kBlock - 1) / kBlock;
+  torch::Tensor out = torch::empty({rows, cols}, input.options().dtype(output_dtype_));
+  // [ceil(M/128), ceil(K/128), 128] with the row inside its 128-row block fastest
+  // (quantization.cc:91-93, quantization.cu:612-621).  Padding rows of the last block stay zero.
+  torch::Tensor scale = torch::zeros({by, bx, kBlock}, input.options().dtype(at::kFloat));
+  quant_call(input, kBlock, eps, out, scale, true);
+  std::optional<torch::Tensor> out_t, scale_t;
+  if (return_transpose) {
+    // Column-wise scales: the same kernel on the transposed matrix.
+    torch::Tensor xt = input.t().contiguous();
+    torch::Tensor ot = torch::empty({cols, rows}, input.options().dtype(output_dtype_));
+    torch::Tensor st = torch::zeros({bx, by, kBlock}, input.options().dtype(at::kFloat));
+    quant_call(xt, kBlock, eps, ot, st, true);
+    out_t = ot;
+    scale_t = st;
+  }
+  return {out, scale, out_t, scale_t};
+}
+
+Quantization::Result Quantization::quantize_square_blockwise(torch::Tensor, bool, float) {
+  TORCH_CHECK(false, "quantize_square_blockwise (128x128 blocks) is not built: the MoE path uses per-row and "
+                     "1x128 scales (quantize_rowwise / quantize_vector_blockwise)");
+  return {};
+}
+
+Quantization::Result Quantization::batch_quantize_square_blockwise(torch::Tensor, bool, float) {
+  TORCH_CHECK(false, "batch_quantize_square_blockwise (128x128 blocks) is not built");
+  return {};
+}
+
+std::tuple<torch::Tensor, torch::Tensor> Quantization::quantize_rowwise(torch::Tensor input, float eps) {
+  TORCH_CHECK(input.dim() == 2, "Input must have 2 dimensions.");
+  FLUX_AMD_CHECK_INPUT(input, input_dtype_);
+  torch::Tensor out = torch::empty(input.sizes(), input.options().dtype(output_dtype_));
+  torch::Tensor scale = torch::empty({input.size(0)}, input.options().dtype(at::kFloat));
+  quant_call(input, 0, eps, out, scale, false);
+  return {out, scale};
+}
+
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor> moe_route_sort(torch::Tensor choosed_experts,
+                                                                                      int64_t nexperts) {
+  FLUX_AMD_CHECK_INPUT(choosed_experts, at::kInt);
+  FLUX_AMD_CHECK_NDIM(choosed_experts, 2);
+  const int32_t ntokens = static_cast<int32_t>(choosed_experts.size(0));
+  const int32_t topk = static_cast<int32_t>(choosed_experts.size(1));
+  TORCH_CHECK(topk >= 1, "topk must be positive");
+  auto iopt = choosed_experts.options();
+  torch::Tensor splits = torch::empty({nexperts}, iopt);
+  torch::Tensor scatter = torch::empty_like(choosed_experts);
+  torch::Tensor gather = torch::empty({static_cast<int64_t>(ntokens) * topk}, iopt);
+  torch::Tensor topk_index = torch::empty({static_cast<int64_t>(ntokens) * topk}, iopt);
+  const size_t ws_bytes = fluxmi_moe_route_sort_workspace_bytes(ntokens, topk, static_cast<int32_t>(nexperts));
+  torch::Tensor ws = torch::empty({static_cast<int64_t>(ws_bytes > 0 ? ws_bytes : 1)}, iopt.dtype(at::kByte));
+  check_status(fluxmi_moe_route_sort(choosed_experts.data_ptr<int32_t>(), ntokens, topk, static_cast<int32_t>(nexperts),
+                                     splits.data_ptr<int32_t>(), nullptr, scatter.data_ptr<int32_t>(),
+                                     gather.data_ptr<int32_t>(), topk_index.data_ptr<int32_t>(), ws.data_ptr(),
+                                     ws_bytes, current_stream()),
+               "fluxmi_moe_route_sort");
+  return {splits, scatter, gather, topk_index};
+}
+
+torch::Tensor calc_scatter_index(torch::Tensor choosed_experts, torch::Tensor splits) {
+  FLUX_AMD_CHECK_INPUT(choosed_experts, at::kInt);
+  FLUX_AMD_CHECK_INPUT(splits, at::kInt);
+  torch::Tensor flat = choosed_experts.dim() == 2 ? choosed_experts : choosed_experts.reshape({-1, 1});
+  // The reference's kernel orders pairs inside an expert by atomics (src/cuda/moe_utils.cu:48-61); this
+  // one returns the stable order, which is one of the orders that kernel may produce.
+  auto r = moe_route_sort(flat, splits.numel());
+  return std::get<1>(r).reshape(choosed_experts.sizes());
+}
+
+torch::Tensor topk_weighted_gather_reduce(std::vector<torch::Tensor> inputs, torch::Tensor routing_idx, int64_t topk,
+                                          std::optional<torch::Tensor> row_weight, double scale) {
+  TORCH_CHECK(!inputs.empty(), "inputs must not be empty");
+  const at::ScalarType st = inputs[0].scalar_type();
+  TORCH_CHECK(st == at::kBFloat16 || st == at::kFloat, "inputs must be bfloat16 or float32");
+  const int64_t m = inputs[0].size(0), n = inputs[0].size(1);
+  TORCH_CHECK(topk >= 1 && m % topk == 0, "rows ", m, " not a multiple of topk ", topk);
+  FLUX_AMD_CHECK_INPUT(routing_idx, at::kInt);
+  TORCH_CHECK(routing_idx.numel() == m, "routing index must have one entry per input row");
+  std::vector<const void *> ptrs;
+  for (auto &t : inputs) {
+    FLUX_AMD_CHECK_INPUT(t, st);
+    FLUX_AMD_CHECK_2D(t, m, n);
+    ptrs.push_back(t.data_ptr());
+  }
+  const float *w = nullptr;
+  if (row_weight.has_value()) {
+    FLUX_AMD_CHECK_INPUT(*row_weight, at::kFloat);
+    TORCH_CHECK(row_weight->numel() == m, "row_weight must be [M]");
+    w = row_weight->data_ptr<float>();
+  }
+  torch::Tensor out = torch::empty({m / topk, n}, inputs[0].options().dtype(at::kBFloat16));
+  check_status(fluxmi_topk_gather_reduce(ptrs.data(), static_cast<int32_t>(ptrs.size()), st == at::kFloat ? 1 : 0,
+                                         routing_idx.data_ptr<int32_t>(), w, static_cast<float>(scale),
+                                         static_cast<int32_t>(m / topk), static_cast<int32_t>(topk),
+                                         static_cast<int32_t>(n), out.data_ptr(), current_stream()),
+               "fluxmi_topk_gather_reduce");
+  return out;
+}
+
+torch::Tensor topk_scatter_reduce(std::vector<torch::Tensor> inputs, torch::Tensor scatter_idx, int64_t topk) {
+  return topk_weighted_gather_reduce(inputs, scatter_idx.reshape({-1}), topk, std::nullopt, 1.0);
+}
+
+bool bitwise_check(torch::Tensor a, torch::Tensor b) {
+  if (a.sizes() != b.sizes() || a.scalar_type() != b.scalar_type()) return false;
+  auto av = a.contiguous().view(at::kByte).reshape({-1});
+  auto bv = b.contiguous().view(at::kByte).reshape({-1});
+  return torch::equal(av, bv);
+}
+
+}  // namespace flux_amd

@@ -1,0 +1,96 @@
+// Declarations of the operator classes and free functions bound in pybind.cc.
+#pragma once
+#include "ths_common.h"
+
+namespace flux_amd {
+
+class GemmGroupedV3AGScatter {
+ public:
+  GemmGroupedV3AGScatter(DistEnvTPWithEP tp_env, MoeArguments moe_args);
+  void clear_buffers();
+  torch::Tensor forward(torch::Tensor inputs_shard, torch::Tensor weights, torch::Tensor splits_gpu,
+                        torch::Tensor scatter_index, std::optional<torch::Tensor> output_scale,
+                        std::optional<torch::Tensor> outputs_buf, std::optional<torch::Tensor> allgather_output,
+                        bool fast_accum, int64_t sm_margin);
+  std::vector<torch::Tensor> forward_multiple_weights(
+      torch::Tensor inputs_shard, std::vector<torch::Tensor> weights, torch::Tensor splits_gpu,
+      torch::Tensor scatter_index, std::optional<std::vector<torch::Tensor>> output_scale,
+      std::optional<std::vector<torch::Tensor>> outputs_buf, std::optional<torch::Tensor> allgather_output,
+      bool fast_accum, int64_t sm_margin);
+
+ private:
+  std::vector<torch::Tensor> forward_impl(torch::Tensor inputs_shard, std::vector<torch::Tensor> weights,
+                                          torch::Tensor splits_gpu, torch::Tensor scatter_index,
+                                          std::optional<std::vector<torch::Tensor>> output_scale,
+                                          std::optional<std::vector<torch::Tensor>> outputs_buf,
+                                          std::optional<torch::Tensor> allgather_output, bool fast_accum,
+                                          int64_t sm_margin);
+  DistEnvTPWithEP tp_env_;
+  MoeArguments moe_args_;
+  torch::Tensor gather_index_;
+};
+
+class GemmGroupedV3GatherRS {
+ public:
+  GemmGroupedV3GatherRS(int64_t total_num_experts, int64_t max_m, int64_t n_dim, int64_t topk, int64_t rank,
+                        int64_t world_size, int64_t tp_world_size, int64_t ep_world_size,
+                        int64_t max_input_groups, bool ep_in_dp);
+  torch::Tensor forward_gather_rs(torch::Tensor input, torch::Tensor weight, torch::Tensor splits_cpu,
+                                  torch::Tensor routing_idx, std::optional<torch::Tensor> n_tokens_per_rank,
+                                  std::optional<torch::Tensor> input_scale,
+                                  std::optional<torch::Tensor> weight_scale,
+                                  std::optional<torch::Tensor> output_vec_scale, bool fast_accum,
+                                  int64_t sm_margin, bool with_stream_sync);
+  torch::Tensor forward_gather_rs_multiple(std::vector<torch::Tensor> inputs, std::vector<torch::Tensor> weights,
+                                           torch::Tensor splits_cpu, torch::Tensor routing_idx,
+                                           std::optional<torch::Tensor> n_tokens_per_rank,
+                                           std::optional<std::vector<torch::Tensor>> input_scale,
+                                           std::optional<std::vector<torch::Tensor>> weight_scale,
+                                           std::optional<std::vector<torch::Tensor>> output_vec_scale,
+                                           bool fast_accum, int64_t sm_margin, bool with_stream_sync);
+  void ep_zero_buffer() {}  // expert-parallel scratch does not exist at world size 1
+
+ private:
+  torch::Tensor forward_impl(std::vector<torch::Tensor> inputs, std::vector<torch::Tensor> weights,
+                             torch::Tensor splits_cpu, torch::Tensor routing_idx,
+                             std::optional<std::vector<torch::Tensor>> input_scale,
+                             std::optional<std::vector<torch::Tensor>> weight_scale,
+                             std::optional<std::vector<torch::Tensor>> output_vec_scale, bool with_stream_sync);
+  void lazy_init(const torch::Tensor &like);
+  int64_t num_experts_, max_m_, n_dim_, topk_, max_input_groups_;
+  bool inter_fp32_ = true;
+  std::vector<torch::Tensor> inter_;
+  torch::Tensor splits_dev_;
+};
+
+class GemmGroupedV3 {
+ public:
+  GemmGroupedV3(torch::Tensor weight, int64_t num_experts);
+  torch::Tensor forward(torch::Tensor input, torch::Tensor splits_cpu);
+
+ private:
+  torch::Tensor weight_;
+};
+
+class Quantization {
+ public:
+  using Result = std::tuple<torch::Tensor, torch::Tensor, std::optional<torch::Tensor>, std::optional<torch::Tensor>>;
+  Quantization(at::ScalarType input_dtype, at::ScalarType output_dtype, int32_t num_streams);
+  Result quantize_vector_blockwise(torch::Tensor input, bool return_transpose, float eps);
+  Result quantize_square_blockwise(torch::Tensor input, bool return_transpose, float eps);
+  Result batch_quantize_square_blockwise(torch::Tensor input, bool return_transpose, float eps);
+  std::tuple<torch::Tensor, torch::Tensor> quantize_rowwise(torch::Tensor input, float eps);
+
+ private:
+  at::ScalarType input_dtype_, output_dtype_;
+};
+
+torch::Tensor calc_scatter_index(torch::Tensor choosed_experts, torch::Tensor splits);
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor> moe_route_sort(torch::Tensor choosed_experts,
+                                                                                      int64_t nexperts);
+torch::Tensor topk_scatter_reduce(std::vector<torch::Tensor> inputs, torch::Tensor scatter_idx, int64_t topk);
+torch::Tensor topk_weighted_gather_reduce(std::vector<torch::Tensor> inputs, torch::Tensor routing_idx,
+                                          int64_t topk, std::optional<torch::Tensor> row_weight, double scale);
+bool bitwise_check(torch::Tensor a, torch::Tensor b);
+
+}  // namespace flux_amd

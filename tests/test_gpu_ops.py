@@ -1,0 +1,158 @@
+"""GPU parity through the operator surface (flux_ths_pybind), written the way the reference's own tests use the
+ops: build the op, call forward, compare with the torch layer (test/python/moe_ag_scatter/test_moe_ag.py:213-311,
+:544-565; test/python/moe_gather_rs/test_moe_gather_rs.py:210-298, :635-648; chaining as in
+examples/moe_flux_only.py:112-131).  bf16 bound: rtol 1e-2 / atol 1e-2 against the fp32 oracle."""
+import numpy as np
+import pytest
+import torch
+
+import flux_amd
+from oracle import configs, layers, quant, routing
+
+pytestmark = pytest.mark.gpu
+RTOL, ATOL = 1e-2, 1e-2
+
+
+def close(got, ref):
+    got = got.float().cpu()
+    bad = (got - ref).abs() > ATOL + RTOL * ref.abs()
+    assert not bool(bad.any()), f"{int(bad.sum())} of {bad.numel()} outside tolerance, max {float((got - ref).abs().max())}"
+
+
+@pytest.fixture(scope="module")
+def c1():
+    return configs.make_workload("C1")
+
+
+def test_routing_functions(c1):
+    wl = c1
+    choosed = wl.choosed.cuda()
+    splits, scatter, gather, tki = flux_amd.moe_route_sort(choosed, wl.experts)
+    assert np.array_equal(splits.cpu().numpy(), wl.splits)
+    assert np.array_equal(scatter.cpu().numpy(), wl.scatter_index)
+    assert np.array_equal(gather.cpu().numpy(), wl.gather_index)
+    assert np.array_equal(tki.cpu().numpy(), wl.topk_index)
+    s2 = flux_amd.calc_scatter_index(choosed, splits)
+    assert flux_amd.bitwise_check(s2, scatter)
+    assert routing.is_gather_index_stable(gather.cpu().numpy(), wl.splits)
+
+
+def test_layer0_layer1_chain_c1(c1):
+    """layer0 forward(outputs_buf=intermediate) -> layer1 forward_gather_rs(routing_idx=scatter_index.view(-1))."""
+    wl = c1
+    t, k, e, h, f = wl.tokens, wl.topk, wl.experts, wl.hidden, wl.ffn
+    x, w1, w2 = (wl.tensors[n].cuda() for n in ("x", "w1", "w2"))
+    splits_gpu = torch.from_numpy(wl.splits).cuda()
+    scatter_index = torch.from_numpy(wl.scatter_index).cuda()
+    tp_env = flux_amd.DistEnvTPWithEP(tp_group=None, nnodes=1, ep_group=None)
+    moe_args = flux_amd.MoeArguments(max_ntokens=t, hidden=h, ffn_hidden=f, nexperts=e, topk=k,
+                                     input_dtype=torch.bfloat16)
+    op0 = flux_amd.GemmGroupedV3AGScatter(tp_env=tp_env, moe_args=moe_args)
+    inter = torch.empty(t * k, f, dtype=torch.bfloat16, device="cuda")
+    ag = torch.empty_like(x)
+    op0.clear_buffers()
+    out0 = op0.forward(inputs_shard=x, weights=w1, splits_gpu=splits_gpu, scatter_index=scatter_index,
+                       outputs_buf=inter, allgather_output=ag, fast_accum=False, sm_margin=0)
+    assert out0.data_ptr() == inter.data_ptr()
+    assert torch.equal(ag, x)
+    close(out0, layers.layer0_fp32(wl.tensors["x"], wl.tensors["w1"], wl.splits, wl.gather_index))
+    # with output_scale; fresh output tensor
+    alpha = (torch.rand(e) + 0.5)
+    out0s = op0.forward(x, w1, splits_gpu, scatter_index, output_scale=alpha.cuda())
+    close(out0s, layers.layer0_fp32(wl.tensors["x"], wl.tensors["w1"], wl.splits, wl.gather_index, alpha))
+    # the reference's own op order (two bf16 roundings) stays within its own bound, 1e-2 / 1.5e-2
+    ref_t = layers.layer0_torch(wl.tensors["x"], wl.tensors["w1"], wl.splits, wl.gather_index, alpha).float()
+    assert torch.allclose(out0s.float().cpu(), ref_t, atol=1e-2, rtol=1.5e-2)
+
+    op1 = flux_amd.GemmGroupedV3GatherRS(total_num_experts=e, max_m=t * k, n_dim=h, topk=k, rank=0, world_size=1,
+                                         tp_world_size=1, ep_world_size=1, max_input_groups=2)
+    splits_cpu = torch.from_numpy(wl.splits)
+    ovs = wl.row_weight.cuda()
+    out1 = op1.forward_gather_rs(input=inter, weight=w2, splits_cpu=splits_cpu, routing_idx=scatter_index.view(-1),
+                                 output_vec_scale=ovs)
+    assert out1.shape == (t, h) and out1.dtype == torch.bfloat16
+    ref1 = layers.layer1_fp32(inter.cpu(), wl.tensors["w2"], wl.splits, wl.scatter_index.reshape(-1), k,
+                              output_vec_scale=wl.row_weight)
+    close(out1, ref1)
+    # scalar input_scale [1] and per-expert weight_scale [E]
+    s_in, s_w = torch.tensor([0.75]), torch.rand(e) + 0.5
+    out1s = op1.forward_gather_rs(inter, w2, splits_cpu, scatter_index.view(-1), input_scale=s_in.cuda(),
+                                  weight_scale=s_w.cuda(), output_vec_scale=ovs, with_stream_sync=True)
+    close(out1s, layers.layer1_fp32(inter.cpu(), wl.tensors["w2"], wl.splits, wl.scatter_index.reshape(-1), k,
+                                    s_in, s_w, wl.row_weight))
+    # two input groups are summed before the reduce
+    out2 = op1.forward_gather_rs_multiple([inter, inter], [w2, w2], splits_cpu, scatter_index.view(-1),
+                                          output_vec_scale=[ovs, ovs])
+    close(out2, 2 * ref1)
+
+
+def test_forward_multiple_weights_and_plain_grouped_gemm(c1):
+    wl = c1
+    x, w1 = wl.tensors["x"].cuda(), wl.tensors["w1"].cuda()
+    w1b = (w1.float() * 0.5).to(torch.bfloat16)
+    op0 = flux_amd.GemmGroupedV3AGScatter(flux_amd.DistEnvTPWithEP(None, 1),
+                                          flux_amd.MoeArguments(wl.tokens, wl.hidden, wl.ffn, wl.experts, wl.topk,
+                                                                torch.bfloat16))
+    outs = op0.forward_multiple_weights(x, [w1, w1b], torch.from_numpy(wl.splits).cuda(),
+                                        torch.from_numpy(wl.scatter_index).cuda())
+    ref = layers.layer0_fp32(wl.tensors["x"], wl.tensors["w1"], wl.splits, wl.gather_index)
+    close(outs[0], ref)
+    close(outs[1], 0.5 * ref)
+    xs = x[torch.from_numpy(wl.gather_index).long().cuda()].contiguous()
+    plain = flux_amd.GemmGroupedV3(w1, wl.experts).forward(xs, torch.from_numpy(wl.splits))
+    assert torch.equal(plain, outs[0])  # same kernel, gather folded in or not: identical bits
+
+
+def test_topk_scatter_reduce_and_shape_errors(c1):
+    wl = c1
+    g = torch.Generator().manual_seed(3)
+    inter = torch.randn(wl.rows, 512, generator=g).to(torch.bfloat16)
+    idx = torch.from_numpy(wl.scatter_index.reshape(-1))
+    out = flux_amd.topk_scatter_reduce([inter.cuda(), inter.cuda()], idx.cuda(), wl.topk)
+    close(out, layers.topk_gather_reduce_fp32([inter, inter], idx.numpy(), wl.topk))
+    op1 = flux_amd.GemmGroupedV3GatherRS(wl.experts, wl.rows, wl.hidden, wl.topk, 0, 1, 1, 1)
+    act, w2 = wl.tensors["act"].cuda(), wl.tensors["w2"].cuda()
+    with pytest.raises(RuntimeError, match="host tensor"):
+        op1.forward_gather_rs(act, w2, torch.from_numpy(wl.splits).cuda(), idx.cuda())
+    with pytest.raises(RuntimeError, match="splits 0-dim mismatch"):
+        op1.forward_gather_rs(act, w2, torch.zeros(3, dtype=torch.int32), idx.cuda())
+    with pytest.raises(RuntimeError, match="routing_idx"):
+        op1.forward_gather_rs(act, w2, torch.from_numpy(wl.splits), idx[:-2].cuda())
+
+
+def test_quantization_op():
+    q = flux_amd.Quantization(torch.bfloat16, torch.float8_e4m3fn)
+    g = torch.Generator().manual_seed(9)
+    x = (torch.randn(200, 384, generator=g) * 3).to(torch.bfloat16)
+    bits = x.view(torch.int16).numpy().view(np.uint16)
+    out, scale, out_t, scale_t = q.quantize_vector_blockwise(x.cuda(), return_tranpose=True)
+    rq, rs = quant.quant_rows_c(bits, 128, 0.0, True)
+    assert out.dtype == torch.float8_e4m3fn and tuple(scale.shape) == (2, 3, 128)
+    assert np.array_equal(out.view(torch.uint8).cpu().numpy(), rq) and np.array_equal(scale.cpu().numpy(), rs)
+    bits_t = np.ascontiguousarray(bits.T)
+    rqt, rst = quant.quant_rows_c(bits_t, 128, 0.0, True)
+    assert tuple(out_t.shape) == (384, 200) and tuple(scale_t.shape) == (3, 2, 128)
+    assert np.array_equal(out_t.view(torch.uint8).cpu().numpy(), rqt) and np.array_equal(scale_t.cpu().numpy(), rst)
+    out2, scale2, none_t, none_s = q.quantize_vector_blockwise(x.cuda(), return_tranpose=False)
+    assert none_t is None and none_s is None and torch.equal(out2.view(torch.uint8), out.view(torch.uint8))
+    qr, sr = q.quantize_rowwise(x.cuda())
+    rq0, rs0 = quant.quant_rows_c(bits)
+    assert np.array_equal(qr.view(torch.uint8).cpu().numpy(), rq0) and np.array_equal(sr.cpu().numpy(), rs0)
+
+
+def test_fp8_layer1_through_ops():
+    """fp8 activations and weights with per-row x per-output-channel scales (weight_scale [E, N], input_scale [M])."""
+    wl = configs.make_workload("C5", tokens=128, hidden=512, ffn=256)
+    e, k = wl.experts, wl.topk
+    q = flux_amd.Quantization(torch.bfloat16, torch.float8_e4m3fn)
+    act, w2 = wl.tensors["act"].cuda(), wl.tensors["w2"].cuda()
+    qa, sa = q.quantize_rowwise(act)
+    qw, sw = q.quantize_rowwise(w2.reshape(-1, wl.ffn))
+    qw, sw = qw.reshape(e, wl.hidden, wl.ffn), sw.reshape(e, wl.hidden)
+    op1 = flux_amd.GemmGroupedV3GatherRS(e, wl.rows, wl.hidden, k, 0, 1, 1, 1)
+    out = op1.forward_gather_rs(qa, qw, torch.from_numpy(wl.splits), torch.from_numpy(wl.scatter_index.reshape(-1)).cuda(),
+                                input_scale=sa, weight_scale=sw, output_vec_scale=wl.row_weight.cuda(), fast_accum=True)
+    z = layers.fp8_grouped_gemm_fp32(qa.cpu(), sa.cpu(), qw.cpu(), sw.cpu(), wl.splits, row_weight=wl.row_weight)
+    ref = layers.topk_gather_reduce_fp32(z, wl.scatter_index.reshape(-1), k)
+    err = float((out.float().cpu() - ref).norm() / ref.norm())
+    assert err < 3e-2, err

@@ -1,0 +1,91 @@
+"""Host logic of the C++ op layer (flux_ths_pybind): names, signatures, defaults and argument errors.
+Runs without a GPU: every check below fires before any kernel launch."""
+import inspect
+
+import pytest
+import torch
+
+import flux_amd
+
+
+def test_module_exports_reference_names():
+    m = flux_amd.flux_ths_pybind
+    for name in ("MoeArguments", "DistEnvTPWithEP", "GemmGroupedV3AGScatter", "GemmGroupedV3GatherRS", "GemmGroupedV3",
+                 "Quantization", "calc_scatter_index", "topk_scatter_reduce", "bitwise_check", "init_flux_shm"):
+        assert hasattr(m, name), name
+        assert getattr(flux_amd, name) is getattr(m, name)
+    for cls, methods in ((m.GemmGroupedV3AGScatter, ("forward", "forward_multiple_weights", "clear_buffers")),
+                         (m.GemmGroupedV3GatherRS, ("forward_gather_rs", "forward_gather_rs_multiple",
+                                                    "forward_gather_rs_no_zerobuffer", "ep_zero_buffer")),
+                         (m.Quantization, ("quantize_vector_blockwise", "quantize_square_blockwise",
+                                           "batch_quantize_square_blockwise"))):
+        for meth in methods:
+            assert hasattr(cls, meth), f"{cls.__name__}.{meth}"
+
+
+def test_keyword_names_match_reference():
+    m = flux_amd.flux_ths_pybind
+    doc = m.GemmGroupedV3AGScatter.forward.__doc__
+    for kw in ("inputs_shard", "weights", "splits_gpu", "scatter_index", "output_scale", "outputs_buf",
+               "allgather_output", "fast_accum", "sm_margin"):
+        assert kw in doc, kw
+    doc = m.GemmGroupedV3GatherRS.forward_gather_rs.__doc__
+    for kw in ("input", "weight", "splits_cpu", "routing_idx", "n_tokens_per_rank", "input_scale", "weight_scale",
+               "output_vec_scale", "fast_accum", "sm_margin", "with_stream_sync"):
+        assert kw in doc, kw
+    assert "return_tranpose" in m.Quantization.quantize_vector_blockwise.__doc__  # the reference's spelling
+    doc = m.GemmGroupedV3GatherRS.__init__.__doc__
+    for kw in ("total_num_experts", "max_m", "n_dim", "topk", "rank", "world_size", "tp_world_size", "ep_world_size",
+               "max_input_groups", "ep_in_dp"):
+        assert kw in doc, kw
+
+
+def test_world_size_above_one_is_rejected():
+    with pytest.raises(RuntimeError, match="one GPU only"):
+        flux_amd.GemmGroupedV3GatherRS(8, 512, 1024, 2, 0, 2, 2, 1)
+    with pytest.raises(RuntimeError, match="one GPU only"):
+        flux_amd.GemmGroupedV3GatherRS(8, 512, 1024, 2, 0, 1, 1, 2)
+
+    class FakeGroup:
+        def __init__(self, n):
+            self.n = n
+
+        def size(self):
+            return self.n
+
+    flux_amd.DistEnvTPWithEP(FakeGroup(1), 1)
+    flux_amd.DistEnvTPWithEP(None, 1, None)
+    with pytest.raises(RuntimeError, match="world size 1"):
+        flux_amd.DistEnvTPWithEP(FakeGroup(8), 1)
+    with pytest.raises(RuntimeError, match="nnodes"):
+        flux_amd.DistEnvTPWithEP(None, 2)
+    flux_amd.init_flux_shm(None)
+
+
+def test_dtype_and_device_checks():
+    with pytest.raises(RuntimeError, match="bfloat16"):
+        flux_amd.Quantization(torch.float16, torch.float8_e4m3fn)
+    with pytest.raises(RuntimeError, match="float8_e4m3fn"):
+        flux_amd.Quantization(torch.bfloat16, torch.float8_e5m2)
+    q = flux_amd.Quantization(torch.bfloat16, torch.float8_e4m3fn)
+    with pytest.raises(RuntimeError, match="2 dimensions"):
+        q.quantize_vector_blockwise(torch.zeros(4, dtype=torch.bfloat16))
+    with pytest.raises(RuntimeError, match="device tensor"):
+        q.quantize_vector_blockwise(torch.zeros(4, 8, dtype=torch.bfloat16))
+    with pytest.raises(RuntimeError, match="not built"):
+        q.quantize_square_blockwise(torch.zeros(4, 8, dtype=torch.bfloat16))
+    args = flux_amd.MoeArguments(max_ntokens=16, hidden=64, ffn_hidden=128, nexperts=4, topk=2,
+                                 input_dtype=torch.bfloat16)
+    assert (args.max_ntokens, args.hidden, args.ffn_hidden, args.nexperts, args.topk) == (16, 64, 128, 4, 2)
+    with pytest.raises(RuntimeError, match="unsupported dtype"):
+        bad = flux_amd.MoeArguments(16, 64, 128, 4, 2, torch.float16)
+        flux_amd.GemmGroupedV3AGScatter(flux_amd.DistEnvTPWithEP(None, 1), bad)
+    with pytest.raises(RuntimeError, match="device tensor"):
+        flux_amd.calc_scatter_index(torch.zeros(4, 2, dtype=torch.int32), torch.zeros(4, dtype=torch.int32))
+    with pytest.raises(RuntimeError, match="device tensor"):
+        flux_amd.topk_scatter_reduce([torch.zeros(8, 8, dtype=torch.bfloat16)], torch.zeros(8, dtype=torch.int32), 2)
+    with pytest.raises(RuntimeError):
+        flux_amd.GemmGroupedV3(torch.zeros(2, 8, 8, dtype=torch.bfloat16), 2)  # host weight
+    assert flux_amd.bitwise_check(torch.arange(6).view(2, 3), torch.arange(6).view(2, 3))
+    assert not flux_amd.bitwise_check(torch.zeros(3), torch.zeros(4))
+    assert not flux_amd.bitwise_check(torch.tensor([0.0]), torch.tensor([-0.0]))
