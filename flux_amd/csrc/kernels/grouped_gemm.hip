@@ -2,7 +2,7 @@
 //
 // Persistent kernel, one 512-thread workgroup (8 waves, 2 per SIMD) per CU, macro tile 256 rows x 256
 // columns, k-step of 64 bytes per row (32 bf16 or 64 fp8).  Both operand tiles are staged in LDS by
-// direct-to-LDS global loads (no register staging) in a 4-deep ring; the row gather of A is folded into
+// direct-to-LDS global loads (no register staging) in a 5-deep ring; the row gather of A is folded into
 // the per-lane global address of those loads.  Each wave owns a 128x64 slice of the macro tile
 // (4x2 MFMA blocks of 32x32, fp32 accumulators).  The two waves that share a SIMD run one phase apart
 // ("ping-pong"): while one issues its LDS fragment reads and the next global loads, the other issues
@@ -12,9 +12,9 @@
 // hardware computes D^T blocks: a lane then holds, for one output row, four consecutive output columns
 // per accumulator quad, which makes the epilogue's stores 8-byte packed bf16x4.
 //
-// Tile schedule: every workgroup rebuilds the per-expert (row offset, tile offset) tables from the
-// device-resident `splits` in LDS, then walks logical tile ids assigned so that the workgroups of one
-// XCD (those with equal blockIdx % 8) take a run of consecutive tiles; tiles of an expert are ordered
+// Tile schedule: every wave walks the device-resident `splits` with scalar loads, in step with the
+// increasing logical tile ids of its workgroup; ids are assigned so that the workgroups of one XCD
+// (those with equal blockIdx % 8) take a run of consecutive tiles; tiles of an expert are ordered
 // column-major (all row tiles of one weight panel first), so an XCD's L2 sees a few weight panels
 // shared by all row tiles of the expert.
 #include "common.hpp"
@@ -25,7 +25,13 @@ namespace {
 constexpr int BM = 256;
 constexpr int BN = 256;
 constexpr int KBYTES = 64;                 // bytes of K per row per k-step
-constexpr int STAGES = 4;
+#ifndef FLUXMI_GEMM_STAGES
+#define FLUXMI_GEMM_STAGES 5
+#endif
+#ifndef FLUXMI_GEMM_ISSUE_FIRST
+#define FLUXMI_GEMM_ISSUE_FIRST 0
+#endif
+constexpr int STAGES = FLUXMI_GEMM_STAGES;  // 5 x 32 KiB = the whole 160 KiB LDS of a CU
 constexpr int DIST = STAGES - 1;           // prefetch distance in k-steps
 constexpr int TILE_BYTES = 256 * KBYTES;   // one operand tile of one stage: 16 KiB
 constexpr int STAGE_BYTES = 2 * TILE_BYTES;
@@ -71,10 +77,6 @@ __device__ __forceinline__ void load_to_lds16(const uint8_t *src, uint8_t *lds_b
   __builtin_amdgcn_global_load_lds((gbl_ptr_t)src, (lds_ptr_t)lds_base, 16, 0, 0);
 }
 
-// LDS tile layout: rows of 64 bytes, two rows per 128-byte line, the eight 16-byte slots of a line
-// xor-swizzled with the line number so that a 32-row column of 16-byte chunks reads without bank
-// conflicts.  Position of (row r, chunk c in 0..3): line = r >> 1, slot = (((r & 1) << 2) | c) ^ (line & 7).
-
 template <int ELT>
 __device__ __forceinline__ f32x16 mfma_step(const i32x4 (&w)[2], const i32x4 (&x)[2], f32x16 acc);
 
@@ -101,11 +103,17 @@ __device__ __forceinline__ f32x16 mfma_step<1>(const i32x4 (&w)[2], const i32x4 
   return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wa, xa, acc, 0, 0, 0, 0, 0, 0);
 }
 
+// Clamped row count of expert e: negative entries count as 0 and rows past max_rows do not exist.
+__device__ __forceinline__ int expert_rows(const GemmParams &p, int e, int row_base) {
+  int rows = p.splits[e];
+  if (rows < 0) rows = 0;
+  if (rows > p.max_rows - row_base) rows = p.max_rows - row_base;
+  return rows;
+}
+
 template <int ELT>
 __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmParams p) {
-  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
-  int32_t *s_row_off = reinterpret_cast<int32_t *>(smem + STAGES * STAGE_BYTES);  // [E + 1]
-  int32_t *s_tile_off = s_row_off + (p.nexperts + 1);                             // [E + 1]
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];  // STAGES x (X tile | W tile)
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: branches on it stay uniform
@@ -116,52 +124,22 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
   const int64_t kbytes = static_cast<int64_t>(p.k) * ELT;
   const int nk = static_cast<int>(kbytes / KBYTES);
 
-  // ---- schedule tables (exclusive prefix sums over experts) ------------------------------------
-  if (wave == 0) {
-    int row_carry = 0, tile_carry = 0;
-    for (int e0 = 0; e0 < p.nexperts; e0 += 64) {
-      const int e = e0 + lane;
-      int rows = e < p.nexperts ? p.splits[e] : 0;
-      if (rows < 0) rows = 0;
-      const int rows_incl = wave_inclusive_scan(rows);
-      // Rows past max_rows do not exist in A / D: clamp the running offsets.
-      int begin = row_carry + rows_incl - rows;
-      int end = row_carry + rows_incl;
-      if (begin > p.max_rows) begin = p.max_rows;
-      if (end > p.max_rows) end = p.max_rows;
-      const int tiles = ((end - begin + BM - 1) / BM) * tiles_n;
-      const int tiles_incl = wave_inclusive_scan(tiles);
-      if (e < p.nexperts) {
-        s_row_off[e] = begin;
-        s_tile_off[e] = tile_carry + tiles_incl - tiles;
-      }
-      row_carry += __shfl(rows_incl, 63, 64);
-      if (row_carry > p.max_rows) row_carry = p.max_rows;
-      tile_carry += __shfl(tiles_incl, 63, 64);
-    }
-    if (lane == 0) {
-      s_row_off[p.nexperts] = row_carry;
-      s_tile_off[p.nexperts] = tile_carry;
-    }
-  }
-  __syncthreads();
-  const int total_tiles = __builtin_amdgcn_readfirstlane(s_tile_off[p.nexperts]);
-
   // ---- per-lane constants -----------------------------------------------------------------------
-  // Direct-to-LDS fill: instruction q (0..15) of a tile covers rows [16q, 16q+16); wave w issues
-  // q = 2w and 2w+1.  Lane l lands in line 8q + (l >> 3), slot l & 7, which holds
-  // row 16q + 2*(l >> 3) + (u >> 2), chunk u & 3 with u = (l & 7) ^ (l >> 3).
-  const int fill_u = (lane & 7) ^ (lane >> 3);
-  const int fill_row = 2 * (lane >> 3) + (fill_u >> 2);  // + 16q
-  const int fill_chunk = fill_u & 3;
+  // LDS tile layout: rows of 64 bytes, four rows per 256-byte "superline" S = r >> 2 (the LDS serves
+  // 64 banks x 4 bytes per clock, 16 lanes of a 16-byte read at a time).  (row r, chunk c) sits in
+  // 16-byte slot ((r & 3) << 2) | (c ^ (S & 3)) of its superline, so the 16 rows read together by a
+  // quarter wave (same chunk) fall into 16 different slots.
+  // Direct-to-LDS fill: instruction q (0..15) of a tile covers rows [16q, 16q+16) = 1 KiB; lane l lands
+  // in superline 4q + (l >> 4), slot l & 15, i.e. row 16q + (l >> 2), chunk (l & 3) ^ ((l >> 4) & 3).
+  const int fill_row = lane >> 2;  // + 16q
+  const int fill_chunk = (lane & 3) ^ ((lane >> 4) & 3);
   // Fragment reads: lane l reads row (l & 31) of a 32-row block, chunk c(s) for s = 0,1.
   int frag_off[2];
 #pragma unroll
   for (int s = 0; s < 2; ++s) {
     const int c = ELT == 2 ? 2 * s + (lane >> 5) : 2 * (lane >> 5) + s;
-    const int line = (lane & 31) >> 1;
-    const int slot = ((((lane & 1) << 2) | c) ^ (line & 7));
-    frag_off[s] = line * 128 + slot * 16;
+    const int slot = ((lane & 3) << 2) | (c ^ ((lane >> 2) & 3));
+    frag_off[s] = ((lane & 31) >> 2) * 256 + slot * 16;
   }
   const int x_frag_base = wm * 128 * KBYTES;                // rows wm*128.. of the X tile
   const int w_frag_base = TILE_BYTES + wn * 64 * KBYTES;    // rows wn*64.. of the W tile
@@ -174,15 +152,42 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
   // Workgroups are dealt to XCDs round-robin; give each XCD a run of consecutive logical tiles.
   const int virt = (grid % 8 == 0) ? (bid & 7) * (grid >> 3) + (bid >> 3) : bid;
 
+  // ---- schedule: walk the experts once, in step with this workgroup's increasing tile ids ----------
+  // All of it is wave-uniform scalar work on the device-resident splits (no LDS, no host round trip).
   int e = 0;
-  for (int tile = virt; tile < total_tiles; tile += grid) {
-    while (tile >= __builtin_amdgcn_readfirstlane(s_tile_off[e + 1])) ++e;
-    const int row_base = __builtin_amdgcn_readfirstlane(s_row_off[e]);
-    const int rows_e = __builtin_amdgcn_readfirstlane(s_row_off[e + 1]) - row_base;
+  int row_base = 0;   // sorted rows before expert e
+  int tile_base = 0;  // tiles before expert e
+  int rows_e = expert_rows(p, 0, 0);
+  int tiles_e = ((rows_e + BM - 1) / BM) * tiles_n;
+
+  int fill_stage = 0;  // ring slot the next issued k-step goes to
+  int read_stage = 0;  // ring slot of the k-step read next
+
+  for (int tile = virt;; tile += grid) {
+    while (e < p.nexperts && tile >= tile_base + tiles_e) {
+      tile_base += tiles_e;
+      row_base += rows_e;
+      ++e;
+      if (e < p.nexperts) {
+        rows_e = expert_rows(p, e, row_base);
+        tiles_e = ((rows_e + BM - 1) / BM) * tiles_n;
+      }
+    }
+    if (e >= p.nexperts) break;
+    // Order inside an expert: row tiles are cut into groups of at most 8; a group is walked
+    // column-major over all weight panels before the next group starts.  32 consecutive tiles (one
+    // XCD's share of a round) then cover about 8 row tiles x 4 panels: 12 distinct operand tiles per
+    // k-step for 32 CUs.
     const int m_tiles = (rows_e + BM - 1) / BM;
-    const int local = tile - __builtin_amdgcn_readfirstlane(s_tile_off[e]);
-    const int nt = local / m_tiles;
-    const int mt = local - nt * m_tiles;
+    const int ngroups_m = (m_tiles + 7) >> 3;
+    const int gm = (m_tiles + ngroups_m - 1) / ngroups_m;  // group height, <= 8
+    const int local = tile - tile_base;
+    const int group = local / (gm * tiles_n);
+    const int group_first = group * gm;
+    const int group_rows = m_tiles - group_first < gm ? m_tiles - group_first : gm;
+    const int in_group = local - group * gm * tiles_n;
+    const int nt = in_group / group_rows;
+    const int mt = group_first + (in_group - nt * group_rows);
     const int m0 = mt * BM;
     const int n0 = nt * BN;
 
@@ -206,7 +211,8 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
     }
 
     auto issue_stage = [&](int kstep) {
-      uint8_t *stage = smem + (kstep % STAGES) * STAGE_BYTES;
+      uint8_t *stage = smem + fill_stage * STAGE_BYTES;
+      fill_stage = fill_stage + 1 == STAGES ? 0 : fill_stage + 1;
       const int64_t koff = static_cast<int64_t>(kstep) * KBYTES;
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
@@ -238,7 +244,10 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
 
     for (int ks = 0; ks < nk; ++ks) {
       // ---- memory phase -------------------------------------------------------------------------
-      const uint8_t *stage = smem + (ks % STAGES) * STAGE_BYTES;
+      const uint8_t *stage = smem + read_stage * STAGE_BYTES;
+      read_stage = read_stage + 1 == STAGES ? 0 : read_stage + 1;
+      const bool more = ks + DIST < nk;
+      if (FLUXMI_GEMM_ISSUE_FIRST && more) issue_stage(ks + DIST);  // global loads first: longest way to go
       i32x4 xf[4][2], wf[2][2];
 #pragma unroll
       for (int j = 0; j < 2; ++j)
@@ -250,8 +259,8 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
 #pragma unroll
         for (int s = 0; s < 2; ++s)
           xf[i][s] = *reinterpret_cast<const i32x4 *>(stage + x_frag_base + i * 32 * KBYTES + frag_off[s]);
-      if (ks + DIST < nk) {
-        issue_stage(ks + DIST);
+      if (!FLUXMI_GEMM_ISSUE_FIRST && more) issue_stage(ks + DIST);
+      if (more) {
         FLUXMI_WAITCNT((DIST - 1) * LOADS_PER_STAGE, 0);  // stage ks+1 landed, fragments in registers
       } else {
         FLUXMI_WAITCNT(0, 0);
@@ -271,8 +280,10 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
       __builtin_amdgcn_sched_barrier(0);
     }
     if (wm == 0) __builtin_amdgcn_s_barrier();  // re-align the two groups
+    // Ring slots skipped by a k loop shorter than the prefetch distance keep both counters in step.
+    if (nk < DIST) read_stage = fill_stage;
 
-    // ---- epilogue: scale, cast, 8-byte stores ---------------------------------------------------
+    // ---- epilogue: scale, cast, packed stores -----------------------------------------------------
     const float tile_scale = scalar * (p.alpha ? p.alpha[e] : 1.f);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -393,9 +404,7 @@ bool mfma_path_ok(const fluxmi_grouped_gemm_args *a) {
          (a->col_scale == nullptr || aligned16(a->col_scale));
 }
 
-size_t mfma_lds_bytes(int nexperts) {
-  return static_cast<size_t>(STAGES) * STAGE_BYTES + 2 * static_cast<size_t>(nexperts + 1) * sizeof(int32_t);
-}
+size_t mfma_lds_bytes() { return static_cast<size_t>(STAGES) * STAGE_BYTES; }
 
 }  // namespace
 }  // namespace fluxmi
@@ -444,7 +453,7 @@ extern "C" int fluxmi_grouped_gemm(const fluxmi_grouped_gemm_args *args, void *,
   FLUXMI_REQUIRE(cus > 0, FLUXMI_ERR_HIP, "grouped_gemm: cannot query the device");
 
   if (mfma_path_ok(args)) {
-    const size_t lds = mfma_lds_bytes(args->nexperts);
+    const size_t lds = mfma_lds_bytes();
     // Upper bound of the tile count: never launch more workgroups than tiles.
     const int64_t tiles_n = (args->n + BN - 1) / BN;
     const int64_t max_tiles = (static_cast<int64_t>(args->max_rows) / BM + args->nexperts) * tiles_n;
