@@ -35,6 +35,8 @@ def parse():
                     help="dtype of the layer1 intermediate [M, H]")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-aux", action="store_true", help="skip the stand-alone HBM kernel measurements")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also run a plain 1 GiB device copy (known traffic) to calibrate rocprofv3 byte counters")
     return ap.parse_args()
 
 
@@ -175,6 +177,13 @@ def main():
             kernels[f"quant_e4m3_{rows}x{cols}"] = {"ms": round(t_q, 4), "gbs": round(b_q / t_q * 1e-6, 1),
                                                     "frac_hbm": round(b_q / t_q * 1e-6 / PEAK_HBM_GBS, 4)}
         del zb
+
+    if a.calib_copy:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        t_cp = time_loop(torch, lambda: dst.copy_(src), 5, warm=1)
+        kernels["calib_copy_1GiB"] = {"ms": round(t_cp, 4), "gbs": round(2 * (1 << 30) / t_cp * 1e-6, 1)}
+        del src, dst
 
     result = {
         "metric": METRIC,
