@@ -23,6 +23,10 @@ METRIC = "grouped-GEMM TFLOP/s (% MFMA peak) + gather-reduce GB/s, Mixtral shape
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
 PEAK_FP8_TFLOPS = 5000.0
 PEAK_HBM_GBS = 8000.0
+# HBM bytes per grouped-GEMM launch on C3 (mean of layer0 and layer1): FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000
+# from the two rocprofv3 --pmc runs summarised in profiles/bench_c3_pmc_counters.md (scale factors from the
+# 1 GiB copy of --calib-copy).  Only valid for the C3 workload with the fp32 layer1 intermediate.
+GEMM_TRAFFIC_C3_BYTES = 3.897e9
 
 
 def parse():
@@ -77,10 +81,10 @@ def time_loop(torch, fn, iters, warm=3):
 
 def cpu_baseline(torch, wl_name, x, w1, w2):
     """The CPU oracle (PyTorch-CPU restatement of the reference's torch layer) on a bounded sample:
-    the first 2048 tokens of the same workload, full hidden / ffn sizes."""
+    one pass over the first `sample_tokens` tokens of the same workload (all of C3), full hidden / ffn sizes."""
     from oracle import configs, layers
 
-    sample_tokens = 2048 if wl_name != "C1" else 256
+    sample_tokens = {"C1": 256, "C3": 8192, "C4": 8192}[wl_name]
     wl, _ = configs.make_routing(wl_name, tokens=sample_tokens)
     threads = torch.get_num_threads()
     xs = x[:sample_tokens].cpu()
@@ -203,7 +207,8 @@ def main():
                    "layer1_intermediate": a.inter,
                    "rows_per_expert_min_max": [int(wl.splits.min()), int(wl.splits.max())]},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
+                     "traffic": GEMM_TRAFFIC_C3_BYTES if (a.workload == "C3" and a.inter == "fp32") else None,
                      "kernel": "grouped_gemm_mfma_kernel<bf16>", "flop_per_launch": gemm_flops,
                      "avg_launch_ms": round(gemm_ms, 4)},
         "kernels": kernels,
