@@ -36,7 +36,6 @@ constexpr int DIST = STAGES - 1;           // prefetch distance in k-steps
 constexpr int TILE_BYTES = 256 * KBYTES;   // one operand tile of one stage: 16 KiB
 constexpr int STAGE_BYTES = 2 * TILE_BYTES;
 constexpr int NTHREADS = 512;
-constexpr int LOADS_PER_STAGE = 4;         // direct-to-LDS instructions per wave per stage
 constexpr int kMaxExperts = 1024;
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -111,46 +110,235 @@ __device__ __forceinline__ int expert_rows(const GemmParams &p, int e, int row_b
   return rows;
 }
 
+// Per-lane constants and ring state shared by all tile shapes.
+struct TileCtx {
+  int wave, lane, wn, wm;
+  int fill_row, fill_chunk;
+  int frag_off[2];
+  int fill_stage;  // ring slot the next issued k-step goes to
+  int read_stage;  // ring slot of the k-step read next
+  int nk;
+  int64_t kbytes;
+  float scalar;
+};
+
+// One output tile of (64*MB) rows x (128*NB) columns: MB x NB MFMA blocks of 32x32 per wave, waves laid
+// out 2 (rows) x 4 (columns).  (MB, NB) = (4, 2) is the 256x256 macro tile; (4, 1), (2, 2) and (2, 1) are
+// the 256x128, 128x256 and 128x128 pieces a tile of the last, partly filled round is cut into.
+template <int ELT, int MB, int NB>
+__device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, TileCtx &c, int e,
+                                          int row_base, int rows_e, int m0, int n0) {
+  constexpr int XLOADS = MB / 2;             // direct-to-LDS instructions per wave per stage, X tile
+  constexpr int WLOADS = NB;                 // same, W tile
+  constexpr int LOADS = XLOADS + WLOADS;
+  const int wave = c.wave, lane = c.lane, wm = c.wm, wn = c.wn, nk = c.nk;
+  const int x_frag_base = wm * (32 * MB) * KBYTES;
+  const int w_frag_base = TILE_BYTES + wn * (32 * NB) * KBYTES;
+
+  // Global source pointers of this lane's fill instructions (k offset added per step).  Instruction q
+  // of a tile covers rows [16q, 16q+16); tail rows re-read the last valid row.
+  const uint8_t *xsrc[XLOADS];
+  const uint8_t *wsrc[WLOADS];
+#pragma unroll
+  for (int j = 0; j < XLOADS; ++j) {
+    int xr = m0 + (XLOADS * wave + j) * 16 + c.fill_row;
+    if (xr > rows_e - 1) xr = rows_e - 1;
+    int64_t arow = row_base + xr;
+    if (p.gather_a) {
+      arow = p.gather_a[arow];
+      if (p.a_rows > 0) arow = arow < 0 ? 0 : (arow >= p.a_rows ? p.a_rows - 1 : arow);
+    }
+    xsrc[j] = p.a + arow * c.kbytes + c.fill_chunk * 16;
+  }
+#pragma unroll
+  for (int j = 0; j < WLOADS; ++j) {
+    int wr = n0 + (WLOADS * wave + j) * 16 + c.fill_row;
+    if (wr > p.n - 1) wr = p.n - 1;
+    wsrc[j] = p.b + (static_cast<int64_t>(e) * p.n + wr) * c.kbytes + c.fill_chunk * 16;
+  }
+
+  auto issue_stage = [&](int kstep) {
+    uint8_t *stage = smem + c.fill_stage * STAGE_BYTES;
+    c.fill_stage = c.fill_stage + 1 == STAGES ? 0 : c.fill_stage + 1;
+    const int64_t koff = static_cast<int64_t>(kstep) * KBYTES;
+#pragma unroll
+    for (int j = 0; j < XLOADS; ++j) load_to_lds16(xsrc[j] + koff, stage + (XLOADS * wave + j) * 1024);
+#pragma unroll
+    for (int j = 0; j < WLOADS; ++j)
+      load_to_lds16(wsrc[j] + koff, stage + TILE_BYTES + (WLOADS * wave + j) * 1024);
+  };
+
+  f32x16 acc[MB][NB];
+#pragma unroll
+  for (int i = 0; i < MB; ++i)
+#pragma unroll
+    for (int j = 0; j < NB; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  // ---- prologue: fill DIST stages ---------------------------------------------------------------
+  FLUXMI_WAITCNT(0, 0);  // stores of the previous tile's epilogue
+#pragma unroll
+  for (int s = 0; s < DIST; ++s)
+    if (s < nk) issue_stage(s);
+  if (nk >= DIST) {
+    FLUXMI_WAITCNT((DIST - 1) * LOADS, 15);
+  } else {
+    FLUXMI_WAITCNT(0, 15);
+  }
+  __builtin_amdgcn_s_barrier();
+  if (wm == 1) __builtin_amdgcn_s_barrier();  // group 1 runs one phase behind group 0
+
+  for (int ks = 0; ks < nk; ++ks) {
+    // ---- memory phase ---------------------------------------------------------------------------
+    const uint8_t *stage = smem + c.read_stage * STAGE_BYTES;
+    c.read_stage = c.read_stage + 1 == STAGES ? 0 : c.read_stage + 1;
+    const bool more = ks + DIST < nk;
+    i32x4 xf[MB][2], wf[NB][2];
+#pragma unroll
+    for (int j = 0; j < NB; ++j)
+#pragma unroll
+      for (int s = 0; s < 2; ++s)
+        wf[j][s] = *reinterpret_cast<const i32x4 *>(stage + w_frag_base + j * 32 * KBYTES + c.frag_off[s]);
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+#pragma unroll
+      for (int s = 0; s < 2; ++s)
+        xf[i][s] = *reinterpret_cast<const i32x4 *>(stage + x_frag_base + i * 32 * KBYTES + c.frag_off[s]);
+    if (more) {
+      issue_stage(ks + DIST);
+      FLUXMI_WAITCNT((DIST - 1) * LOADS, 0);  // stage ks+1 landed, fragments in registers
+    } else {
+      FLUXMI_WAITCNT(0, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- compute phase --------------------------------------------------------------------------
+    __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+#pragma unroll
+      for (int j = 0; j < NB; ++j) acc[i][j] = mfma_step<ELT>(wf[j], xf[i], acc[i][j]);
+    __builtin_amdgcn_s_setprio(0);
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  if (wm == 0) __builtin_amdgcn_s_barrier();  // re-align the two groups
+
+  // ---- epilogue: scale, cast, packed stores -------------------------------------------------------
+  const float tile_scale = c.scalar * (p.alpha ? p.alpha[e] : 1.f);
+#pragma unroll
+  for (int i = 0; i < MB; ++i) {
+    const int m = m0 + wm * (32 * MB) + i * 32 + (lane & 31);
+    if (m >= rows_e) continue;
+    const int64_t srow = row_base + m;
+    const float rs = tile_scale * (p.row_scale ? p.row_scale[srow] : 1.f);
+    int64_t drow = srow;
+    if (p.scatter_d) {
+      drow = p.scatter_d[srow];
+      if (drow < 0 || drow >= p.max_rows) continue;
+    }
+    uint16_t *dptr = static_cast<uint16_t *>(p.d) + drow * p.n;
+    float *dptr32 = static_cast<float *>(p.d) + drow * p.n;
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int n = n0 + wn * (32 * NB) + j * 32 + q * 8 + (lane >> 5) * 4;
+        if (n >= p.n) continue;  // n % 4 == 0 is required, so a quad is all in or all out
+        float v0 = acc[i][j][4 * q + 0] * rs;
+        float v1 = acc[i][j][4 * q + 1] * rs;
+        float v2 = acc[i][j][4 * q + 2] * rs;
+        float v3 = acc[i][j][4 * q + 3] * rs;
+        if (p.col_scale) {
+          const float4 cs = *reinterpret_cast<const float4 *>(p.col_scale + static_cast<int64_t>(e) * p.n + n);
+          v0 *= cs.x;
+          v1 *= cs.y;
+          v2 *= cs.z;
+          v3 *= cs.w;
+        }
+        if (p.d_fp32) {
+          *reinterpret_cast<float4 *>(dptr32 + n) = make_float4(v0, v1, v2, v3);
+        } else {
+          u32x2 o;
+          o[0] = float_to_bf16_bits(v0) | (static_cast<uint32_t>(float_to_bf16_bits(v1)) << 16);
+          o[1] = float_to_bf16_bits(v2) | (static_cast<uint32_t>(float_to_bf16_bits(v3)) << 16);
+          *reinterpret_cast<u32x2 *>(dptr + n) = o;
+        }
+      }
+    }
+  }
+}
+
 template <int ELT>
 __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmParams p) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];  // STAGES x (X tile | W tile)
 
+  TileCtx c;
   const int tid = threadIdx.x;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: branches on it stay uniform
-  const int lane = tid & 63;
-  const int wn = wave & 3;   // 64-column slice
-  const int wm = wave >> 2;  // 128-row slice == ping-pong group
+  c.wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: branches on it stay uniform
+  c.lane = tid & 63;
+  c.wn = c.wave & 3;   // column slice
+  c.wm = c.wave >> 2;  // row slice == ping-pong group
+  const int lane = c.lane;
   const int tiles_n = (p.n + BN - 1) / BN;
-  const int64_t kbytes = static_cast<int64_t>(p.k) * ELT;
-  const int nk = static_cast<int>(kbytes / KBYTES);
+  c.kbytes = static_cast<int64_t>(p.k) * ELT;
+  c.nk = static_cast<int>(c.kbytes / KBYTES);
 
-  // ---- per-lane constants -----------------------------------------------------------------------
   // LDS tile layout: rows of 64 bytes, four rows per 256-byte "superline" S = r >> 2 (the LDS serves
   // 64 banks x 4 bytes per clock, 16 lanes of a 16-byte read at a time).  (row r, chunk c) sits in
   // 16-byte slot ((r & 3) << 2) | (c ^ (S & 3)) of its superline, so the 16 rows read together by a
   // quarter wave (same chunk) fall into 16 different slots.
-  // Direct-to-LDS fill: instruction q (0..15) of a tile covers rows [16q, 16q+16) = 1 KiB; lane l lands
-  // in superline 4q + (l >> 4), slot l & 15, i.e. row 16q + (l >> 2), chunk (l & 3) ^ ((l >> 4) & 3).
-  const int fill_row = lane >> 2;  // + 16q
-  const int fill_chunk = (lane & 3) ^ ((lane >> 4) & 3);
+  // Direct-to-LDS fill: instruction q of a tile covers rows [16q, 16q+16) = 1 KiB; lane l lands in
+  // superline 4q + (l >> 4), slot l & 15, i.e. row 16q + (l >> 2), chunk (l & 3) ^ ((l >> 4) & 3).
+  c.fill_row = lane >> 2;
+  c.fill_chunk = (lane & 3) ^ ((lane >> 4) & 3);
   // Fragment reads: lane l reads row (l & 31) of a 32-row block, chunk c(s) for s = 0,1.
-  int frag_off[2];
 #pragma unroll
   for (int s = 0; s < 2; ++s) {
-    const int c = ELT == 2 ? 2 * s + (lane >> 5) : 2 * (lane >> 5) + s;
-    const int slot = ((lane & 3) << 2) | (c ^ ((lane >> 2) & 3));
-    frag_off[s] = ((lane & 31) >> 2) * 256 + slot * 16;
+    const int ch = ELT == 2 ? 2 * s + (lane >> 5) : 2 * (lane >> 5) + s;
+    const int slot = ((lane & 3) << 2) | (ch ^ ((lane >> 2) & 3));
+    c.frag_off[s] = ((lane & 31) >> 2) * 256 + slot * 16;
   }
-  const int x_frag_base = wm * 128 * KBYTES;                // rows wm*128.. of the X tile
-  const int w_frag_base = TILE_BYTES + wn * 64 * KBYTES;    // rows wn*64.. of the W tile
-
-  float scalar = p.scalar;
-  if (p.scalar_dev) scalar *= p.scalar_dev[0];
+  c.scalar = p.scalar;
+  if (p.scalar_dev) c.scalar *= p.scalar_dev[0];
+  c.fill_stage = 0;
+  c.read_stage = 0;
 
   const int grid = gridDim.x;
   const int bid = blockIdx.x;
-  // Workgroups are dealt to XCDs round-robin; give each XCD a run of consecutive logical tiles.
+  // Workgroups are dealt to XCDs round-robin; give each XCD a run of consecutive logical work items.
   const int virt = (grid % 8 == 0) ? (bid & 7) * (grid >> 3) + (bid >> 3) : bid;
+
+  // ---- total tile count (one wave-wide pass over splits) -> shape of the last round -----------------
+  int total_tiles = 0;
+  {
+    int row_carry = 0, acc_tiles = 0;
+    for (int e0 = 0; e0 < p.nexperts; e0 += 64) {
+      const int ee = e0 + lane;
+      int rows = ee < p.nexperts ? p.splits[ee] : 0;
+      if (rows < 0) rows = 0;
+      const int incl = wave_inclusive_scan(rows);
+      int begin = row_carry + incl - rows, end = row_carry + incl;
+      if (begin > p.max_rows) begin = p.max_rows;
+      if (end > p.max_rows) end = p.max_rows;
+      int tiles = ((end - begin + BM - 1) / BM) * tiles_n;
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) tiles += __shfl_xor(tiles, off, 64);
+      acc_tiles += tiles;
+      row_carry += __shfl(incl, 63, 64);
+    }
+    total_tiles = __builtin_amdgcn_readfirstlane(acc_tiles);
+  }
+  // Full rounds run whole 256x256 tiles.  The tiles of the last, partly filled round are cut into
+  // `pieces` parts (4: 128x128, 2: 256x128) when that still fits one round, so that the chip does not
+  // idle while a fraction of the CUs finishes whole tiles.
+  const int full_items = (total_tiles / grid) * grid;
+  const int rem_tiles = total_tiles - full_items;
+  const int pieces = rem_tiles * 4 <= grid ? 4 : (rem_tiles * 2 <= grid ? 2 : 1);
+  const int total_items = full_items + rem_tiles * pieces;
 
   // ---- schedule: walk the experts once, in step with this workgroup's increasing tile ids ----------
   // All of it is wave-uniform scalar work on the device-resident splits (no LDS, no host round trip).
@@ -160,10 +348,12 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
   int rows_e = expert_rows(p, 0, 0);
   int tiles_e = ((rows_e + BM - 1) / BM) * tiles_n;
 
-  int fill_stage = 0;  // ring slot the next issued k-step goes to
-  int read_stage = 0;  // ring slot of the k-step read next
-
-  for (int tile = virt;; tile += grid) {
+  for (int item = virt; item < total_items; item += grid) {
+    int tile = item, piece = 0;
+    if (item >= full_items) {
+      tile = full_items + (item - full_items) / pieces;
+      piece = (item - full_items) % pieces;
+    }
     while (e < p.nexperts && tile >= tile_base + tiles_e) {
       tile_base += tiles_e;
       row_base += rows_e;
@@ -188,144 +378,18 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
     const int in_group = local - group * gm * tiles_n;
     const int nt = in_group / group_rows;
     const int mt = group_first + (in_group - nt * group_rows);
-    const int m0 = mt * BM;
-    const int n0 = nt * BN;
+    int m0 = mt * BM;
+    int n0 = nt * BN;
 
-    // Global source pointers of this lane's 2 + 2 fill instructions (k offset added per step).
-    const uint8_t *xsrc[2];
-    const uint8_t *wsrc[2];
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int r = (2 * wave + j) * 16 + fill_row;
-      int xr = m0 + r;
-      if (xr > rows_e - 1) xr = rows_e - 1;  // tail rows re-read the last valid row
-      int64_t arow = row_base + xr;
-      if (p.gather_a) {
-        arow = p.gather_a[arow];
-        if (p.a_rows > 0) arow = arow < 0 ? 0 : (arow >= p.a_rows ? p.a_rows - 1 : arow);
-      }
-      xsrc[j] = p.a + arow * kbytes + fill_chunk * 16;
-      int wr = n0 + r;
-      if (wr > p.n - 1) wr = p.n - 1;
-      wsrc[j] = p.b + (static_cast<int64_t>(e) * p.n + wr) * kbytes + fill_chunk * 16;
-    }
-
-    auto issue_stage = [&](int kstep) {
-      uint8_t *stage = smem + fill_stage * STAGE_BYTES;
-      fill_stage = fill_stage + 1 == STAGES ? 0 : fill_stage + 1;
-      const int64_t koff = static_cast<int64_t>(kstep) * KBYTES;
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        load_to_lds16(xsrc[j] + koff, stage + (2 * wave + j) * 1024);
-        load_to_lds16(wsrc[j] + koff, stage + TILE_BYTES + (2 * wave + j) * 1024);
-      }
-    };
-
-    f32x16 acc[4][2];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int j = 0; j < 2; ++j)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
-
-    // ---- prologue: fill DIST stages -------------------------------------------------------------
-    FLUXMI_WAITCNT(0, 0);  // stores of the previous tile's epilogue
-#pragma unroll
-    for (int s = 0; s < DIST; ++s)
-      if (s < nk) issue_stage(s);
-    if (nk >= DIST) {
-      FLUXMI_WAITCNT((DIST - 1) * LOADS_PER_STAGE, 15);
+    if (item < full_items || pieces == 1) {
+      gemm_tile<ELT, 4, 2>(p, smem, c, e, row_base, rows_e, m0, n0);
+    } else if (pieces == 2) {
+      n0 += piece * 128;
+      if (n0 < p.n) gemm_tile<ELT, 4, 1>(p, smem, c, e, row_base, rows_e, m0, n0);
     } else {
-      FLUXMI_WAITCNT(0, 15);
-    }
-    __builtin_amdgcn_s_barrier();
-    if (wm == 1) __builtin_amdgcn_s_barrier();  // group 1 runs one phase behind group 0
-
-    for (int ks = 0; ks < nk; ++ks) {
-      // ---- memory phase -------------------------------------------------------------------------
-      const uint8_t *stage = smem + read_stage * STAGE_BYTES;
-      read_stage = read_stage + 1 == STAGES ? 0 : read_stage + 1;
-      const bool more = ks + DIST < nk;
-      if (FLUXMI_GEMM_ISSUE_FIRST && more) issue_stage(ks + DIST);  // global loads first: longest way to go
-      i32x4 xf[4][2], wf[2][2];
-#pragma unroll
-      for (int j = 0; j < 2; ++j)
-#pragma unroll
-        for (int s = 0; s < 2; ++s)
-          wf[j][s] = *reinterpret_cast<const i32x4 *>(stage + w_frag_base + j * 32 * KBYTES + frag_off[s]);
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int s = 0; s < 2; ++s)
-          xf[i][s] = *reinterpret_cast<const i32x4 *>(stage + x_frag_base + i * 32 * KBYTES + frag_off[s]);
-      if (!FLUXMI_GEMM_ISSUE_FIRST && more) issue_stage(ks + DIST);
-      if (more) {
-        FLUXMI_WAITCNT((DIST - 1) * LOADS_PER_STAGE, 0);  // stage ks+1 landed, fragments in registers
-      } else {
-        FLUXMI_WAITCNT(0, 0);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-      __builtin_amdgcn_s_barrier();
-      __builtin_amdgcn_sched_barrier(0);
-      // ---- compute phase ------------------------------------------------------------------------
-      __builtin_amdgcn_s_setprio(1);
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = mfma_step<ELT>(wf[j], xf[i], acc[i][j]);
-      __builtin_amdgcn_s_setprio(0);
-      __builtin_amdgcn_sched_barrier(0);
-      __builtin_amdgcn_s_barrier();
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    if (wm == 0) __builtin_amdgcn_s_barrier();  // re-align the two groups
-    // Ring slots skipped by a k loop shorter than the prefetch distance keep both counters in step.
-    if (nk < DIST) read_stage = fill_stage;
-
-    // ---- epilogue: scale, cast, packed stores -----------------------------------------------------
-    const float tile_scale = scalar * (p.alpha ? p.alpha[e] : 1.f);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int m = m0 + wm * 128 + i * 32 + (lane & 31);
-      if (m >= rows_e) continue;
-      const int64_t srow = row_base + m;
-      const float rs = tile_scale * (p.row_scale ? p.row_scale[srow] : 1.f);
-      int64_t drow = srow;
-      if (p.scatter_d) {
-        drow = p.scatter_d[srow];
-        if (drow < 0 || drow >= p.max_rows) continue;
-      }
-      uint16_t *dptr = static_cast<uint16_t *>(p.d) + drow * p.n;
-      float *dptr32 = static_cast<float *>(p.d) + drow * p.n;
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int n = n0 + wn * 64 + j * 32 + q * 8 + (lane >> 5) * 4;
-          if (n >= p.n) continue;  // n % 4 == 0 is required, so a quad is all in or all out
-          float v0 = acc[i][j][4 * q + 0] * rs;
-          float v1 = acc[i][j][4 * q + 1] * rs;
-          float v2 = acc[i][j][4 * q + 2] * rs;
-          float v3 = acc[i][j][4 * q + 3] * rs;
-          if (p.col_scale) {
-            const float4 cs =
-                *reinterpret_cast<const float4 *>(p.col_scale + static_cast<int64_t>(e) * p.n + n);
-            v0 *= cs.x;
-            v1 *= cs.y;
-            v2 *= cs.z;
-            v3 *= cs.w;
-          }
-          if (p.d_fp32) {
-            *reinterpret_cast<float4 *>(dptr32 + n) = make_float4(v0, v1, v2, v3);
-          } else {
-            u32x2 o;
-            o[0] = float_to_bf16_bits(v0) | (static_cast<uint32_t>(float_to_bf16_bits(v1)) << 16);
-            o[1] = float_to_bf16_bits(v2) | (static_cast<uint32_t>(float_to_bf16_bits(v3)) << 16);
-            *reinterpret_cast<u32x2 *>(dptr + n) = o;
-          }
-        }
-      }
+      m0 += (piece >> 1) * 128;
+      n0 += (piece & 1) * 128;
+      if (m0 < rows_e && n0 < p.n) gemm_tile<ELT, 2, 1>(p, smem, c, e, row_base, rows_e, m0, n0);
     }
   }
 }
