@@ -10,7 +10,11 @@ namespace fluxmi {
 namespace {
 
 constexpr int kMaxGroups = 4;
-constexpr int kThreads = 256;
+constexpr int kMaxThreads = 512;
+// Inputs up to this size are read with ordinary loads: they were just written by the grouped GEMM and a
+// good part of them still sits in the 256 MiB Infinity Cache, which non-temporal loads do not use as well.
+// Larger inputs stream from HBM and are read non-temporally (measured: +10 % either way).
+constexpr size_t kPlainLoadMaxBytes = size_t{288} << 20;
 
 struct GroupPtrs {
   const void *p[kMaxGroups];
@@ -24,15 +28,21 @@ struct Vec8 {
   u32x4 v[IN_F32 ? 2 : 1];
 };
 
-template <bool IN_F32>
+template <bool NT>
+__device__ __forceinline__ u32x4 load16(const u32x4 *src) {
+  if constexpr (NT) return __builtin_nontemporal_load(src);
+  else return *src;
+}
+
+template <bool IN_F32, bool NT>
 __device__ __forceinline__ Vec8<IN_F32> load8(const void *base, size_t row, size_t row_vecs, int v) {
   Vec8<IN_F32> r;
   if constexpr (IN_F32) {
     const u32x4 *src = reinterpret_cast<const u32x4 *>(base) + (row * row_vecs + v) * 2;
-    r.v[0] = __builtin_nontemporal_load(src);
-    r.v[1] = __builtin_nontemporal_load(src + 1);
+    r.v[0] = load16<NT>(src);
+    r.v[1] = load16<NT>(src + 1);
   } else {
-    r.v[0] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(base) + row * row_vecs + v);
+    r.v[0] = load16<NT>(reinterpret_cast<const u32x4 *>(base) + row * row_vecs + v);
   }
   return r;
 }
@@ -61,15 +71,17 @@ __device__ __forceinline__ void accumulate8(float (&acc)[8], const Vec8<false> &
 }
 
 // TOPK > 0: compile-time top-k (loads fully unrolled).  TOPK == 0: run-time top-k.
-template <int TOPK, int NGROUPS, bool WEIGHTED, bool IN_F32>
-__global__ __launch_bounds__(kThreads) void topk_gather_reduce_kernel(
-    GroupPtrs in, const int32_t *__restrict__ routing_idx, const float *__restrict__ row_weight,
-    float scale, int32_t topk_rt, int32_t nvec /* n / 8 */, uint16_t *__restrict__ out) {
+// NT: non-temporal source loads.  The choice is made once per launch and hoisted out of the load
+// sequence, so that no control flow sits between the loads of one output vector.
+template <int TOPK, int NGROUPS, bool WEIGHTED, bool IN_F32, bool NT>
+__device__ __forceinline__ void topk_gather_reduce_body(
+    const GroupPtrs &in, const int32_t *__restrict__ routing_idx, const float *__restrict__ row_weight,
+    float scale, int32_t topk_rt, int32_t nvec, uint16_t *__restrict__ out) {
   const int t = blockIdx.x;
   const int topk = TOPK > 0 ? TOPK : topk_rt;
   const size_t row_vecs = static_cast<size_t>(nvec);
-
-  for (int v = blockIdx.y * kThreads + threadIdx.x; v < nvec; v += gridDim.y * kThreads) {
+  const int nthreads = blockDim.x;
+  for (int v = blockIdx.y * nthreads + threadIdx.x; v < nvec; v += gridDim.y * nthreads) {
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     if constexpr (TOPK > 0) {
       Vec8<IN_F32> vals[NGROUPS][TOPK];
@@ -83,7 +95,7 @@ __global__ __launch_bounds__(kThreads) void topk_gather_reduce_kernel(
         for (int g = 0; g < NGROUPS; ++g) {
           vals[g][j] = zero8<IN_F32>();
           // r is wave-uniform: a skipped (dropped) row costs no traffic
-          if (r >= 0) vals[g][j] = load8<IN_F32>(in.p[g], static_cast<size_t>(r), row_vecs, v);
+          if (r >= 0) vals[g][j] = load8<IN_F32, NT>(in.p[g], static_cast<size_t>(r), row_vecs, v);
         }
       }
 #pragma unroll
@@ -97,7 +109,7 @@ __global__ __launch_bounds__(kThreads) void topk_gather_reduce_kernel(
           const int32_t r = routing_idx[static_cast<size_t>(t) * topk + j];
           if (r < 0) continue;
           const float w = WEIGHTED ? row_weight[r] : 1.f;
-          accumulate8(acc, load8<IN_F32>(in.p[g], static_cast<size_t>(r), row_vecs, v), w);
+          accumulate8(acc, load8<IN_F32, NT>(in.p[g], static_cast<size_t>(r), row_vecs, v), w);
         }
       }
     }
@@ -113,12 +125,25 @@ __global__ __launch_bounds__(kThreads) void topk_gather_reduce_kernel(
   }
 }
 
+template <int TOPK, int NGROUPS, bool WEIGHTED, bool IN_F32>
+__global__ __launch_bounds__(kMaxThreads) void topk_gather_reduce_kernel(
+    GroupPtrs in, const int32_t *__restrict__ routing_idx, const float *__restrict__ row_weight,
+    float scale, int32_t topk_rt, int32_t nvec /* n / 8 */, int32_t nt_loads,
+    uint16_t *__restrict__ out) {
+  if (nt_loads)
+    topk_gather_reduce_body<TOPK, NGROUPS, WEIGHTED, IN_F32, true>(in, routing_idx, row_weight, scale, topk_rt,
+                                                                   nvec, out);
+  else
+    topk_gather_reduce_body<TOPK, NGROUPS, WEIGHTED, IN_F32, false>(in, routing_idx, row_weight, scale, topk_rt,
+                                                                    nvec, out);
+}
+
 template <int TOPK, int NGROUPS>
-void launch(bool weighted, bool in_f32, dim3 grid, hipStream_t s, const GroupPtrs &in,
+void launch(bool weighted, bool in_f32, dim3 grid, int threads, int nt, hipStream_t s, const GroupPtrs &in,
             const int32_t *idx, const float *w, float scale, int32_t topk, int32_t nvec, uint16_t *out) {
-#define FLUXMI_GR_LAUNCH(W, F)                                                                        \
-  hipLaunchKernelGGL((topk_gather_reduce_kernel<TOPK, NGROUPS, W, F>), grid, dim3(kThreads), 0, s, in, \
-                     idx, w, scale, topk, nvec, out)
+#define FLUXMI_GR_LAUNCH(W, F)                                                                       \
+  hipLaunchKernelGGL((topk_gather_reduce_kernel<TOPK, NGROUPS, W, F>), grid, dim3(threads), 0, s, in, \
+                     idx, w, scale, topk, nvec, nt, out)
   if (weighted) {
     if (in_f32) FLUXMI_GR_LAUNCH(true, true);
     else FLUXMI_GR_LAUNCH(true, false);
@@ -130,15 +155,15 @@ void launch(bool weighted, bool in_f32, dim3 grid, hipStream_t s, const GroupPtr
 }
 
 template <int NGROUPS>
-void dispatch_topk(bool weighted, bool in_f32, dim3 grid, hipStream_t s, const GroupPtrs &in, const int32_t *idx,
+void dispatch_topk(bool weighted, bool in_f32, dim3 grid, int threads, int nt, hipStream_t s, const GroupPtrs &in, const int32_t *idx,
                    const float *w, float scale, int32_t topk, int32_t nvec, uint16_t *out) {
   switch (topk) {
-    case 1: launch<1, NGROUPS>(weighted, in_f32, grid, s, in, idx, w, scale, topk, nvec, out); break;
-    case 2: launch<2, NGROUPS>(weighted, in_f32, grid, s, in, idx, w, scale, topk, nvec, out); break;
-    case 4: launch<4, NGROUPS>(weighted, in_f32, grid, s, in, idx, w, scale, topk, nvec, out); break;
-    case 6: launch<6, NGROUPS>(weighted, in_f32, grid, s, in, idx, w, scale, topk, nvec, out); break;
-    case 8: launch<8, NGROUPS>(weighted, in_f32, grid, s, in, idx, w, scale, topk, nvec, out); break;
-    default: launch<0, NGROUPS>(weighted, in_f32, grid, s, in, idx, w, scale, topk, nvec, out); break;
+    case 1: launch<1, NGROUPS>(weighted, in_f32, grid, threads, nt, s, in, idx, w, scale, topk, nvec, out); break;
+    case 2: launch<2, NGROUPS>(weighted, in_f32, grid, threads, nt, s, in, idx, w, scale, topk, nvec, out); break;
+    case 4: launch<4, NGROUPS>(weighted, in_f32, grid, threads, nt, s, in, idx, w, scale, topk, nvec, out); break;
+    case 6: launch<6, NGROUPS>(weighted, in_f32, grid, threads, nt, s, in, idx, w, scale, topk, nvec, out); break;
+    case 8: launch<8, NGROUPS>(weighted, in_f32, grid, threads, nt, s, in, idx, w, scale, topk, nvec, out); break;
+    default: launch<0, NGROUPS>(weighted, in_f32, grid, threads, nt, s, in, idx, w, scale, topk, nvec, out); break;
   }
 }
 
@@ -173,20 +198,23 @@ extern "C" int fluxmi_topk_gather_reduce(const void *const *in, int32_t ngroups,
   const int32_t nvec = n / 8;
   // One workgroup per token row; rows wider than 2 vectors per lane are split over blockIdx.y so
   // that small token counts still fill the chip.
+  const int threads = nvec >= 512 ? 512 : 256;
   int ysplit = 1;
   if (ntokens < 2048) {
-    ysplit = (nvec + kThreads - 1) / kThreads;
+    ysplit = (nvec + threads - 1) / threads;
     if (ysplit > 16) ysplit = 16;
   }
+  const size_t in_bytes = static_cast<size_t>(ntokens) * topk * n * (in_fp32 ? 4 : 2) * ngroups;
+  const int nt = in_bytes > kPlainLoadMaxBytes ? 1 : 0;
   const dim3 grid(static_cast<unsigned>(ntokens), static_cast<unsigned>(ysplit));
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool weighted = row_weight != nullptr;
   uint16_t *o = static_cast<uint16_t *>(out);
   switch (ngroups) {
-    case 1: dispatch_topk<1>(weighted, in_fp32 != 0, grid, s, gp, routing_idx, row_weight, scale, topk, nvec, o); break;
-    case 2: dispatch_topk<2>(weighted, in_fp32 != 0, grid, s, gp, routing_idx, row_weight, scale, topk, nvec, o); break;
-    case 3: dispatch_topk<3>(weighted, in_fp32 != 0, grid, s, gp, routing_idx, row_weight, scale, topk, nvec, o); break;
-    default: dispatch_topk<4>(weighted, in_fp32 != 0, grid, s, gp, routing_idx, row_weight, scale, topk, nvec, o); break;
+    case 1: dispatch_topk<1>(weighted, in_fp32 != 0, grid, threads, nt, s, gp, routing_idx, row_weight, scale, topk, nvec, o); break;
+    case 2: dispatch_topk<2>(weighted, in_fp32 != 0, grid, threads, nt, s, gp, routing_idx, row_weight, scale, topk, nvec, o); break;
+    case 3: dispatch_topk<3>(weighted, in_fp32 != 0, grid, threads, nt, s, gp, routing_idx, row_weight, scale, topk, nvec, o); break;
+    default: dispatch_topk<4>(weighted, in_fp32 != 0, grid, threads, nt, s, gp, routing_idx, row_weight, scale, topk, nvec, o); break;
   }
   FLUXMI_HIP_CHECK(hipGetLastError());
   return FLUXMI_OK;
