@@ -2,6 +2,8 @@
 // gather_index, topk_index.
 //
 // The flat pair array is cut into chunks of kChunk = 512 pairs, one wave per chunk (8 wave-steps of 64).
+// Inputs of up to 65536 pairs and 512 experts run the same three steps inside one workgroup
+// (route_sort_single_kernel); larger ones take three launches:
 //   1. route_hist_kernel    per-chunk expert histogram in LDS (ds_add_u32), written to hist[chunk][e]
 //   2. route_scan_kernel    one wave per expert: exclusive scan of hist[:, e] over chunks (wave scan),
 //                           in place; the total is splits[e]
@@ -69,6 +71,61 @@ __global__ __launch_bounds__(kThreads) void route_scan_kernel(int32_t *__restric
   }
 }
 
+// Stable scatter of the pairs [first, first + 64*steps) by one wave.  running[e] holds the next free
+// sorted row of expert e for this range (LDS, private to the wave).  Per wave-step the lanes holding the
+// same expert are found with one ballot per id bit, ranked with mbcnt, and the first of them advances
+// running[e].
+template <bool STAGED>
+__device__ __forceinline__ void scatter_range(const int32_t *__restrict__ choosed, const uint16_t *staged,
+                                              int first, int steps,
+                                              int32_t npairs, int32_t topk, int32_t nexperts, int32_t idbits,
+                                              int32_t *running, int32_t *__restrict__ scatter_index,
+                                              int32_t *__restrict__ gather_index,
+                                              int32_t *__restrict__ topk_index) {
+  const int lane = threadIdx.x & 63;
+  // Expert ids are fetched several wave-steps at a time.  From global memory all 8 steps of a chunk are
+  // fetched before the first store: vmcnt counts loads and stores in one queue, so a later load would
+  // also wait for every store issued before it.
+  constexpr int kAhead = STAGED ? 4 : 8;
+  int32_t ids[kAhead];
+  for (int s = 0; s < steps; ++s) {
+    if ((s & (kAhead - 1)) == 0) {
+#pragma unroll
+      for (int a = 0; a < kAhead; ++a) {
+        const int ia = first + (s + a) * 64 + lane;
+        if constexpr (STAGED) ids[a] = (s + a < steps && ia < npairs) ? static_cast<int32_t>(staged[ia]) : -1;
+        else ids[a] = (s + a < steps && ia < npairs) ? choosed[ia] : -1;
+      }
+    }
+    const int i = first + s * 64 + lane;
+    int32_t e = ids[0];
+#pragma unroll
+    for (int a = 1; a < kAhead; ++a)
+      if ((s & (kAhead - 1)) == a) e = ids[a];
+    if (e < 0 || e >= nexperts) e = -1;
+    // Lanes that hold the same expert id as this lane.
+    uint64_t same = __ballot(e >= 0);
+    for (int b = 0; b < idbits; ++b) {
+      const uint64_t bit = __ballot((e >> b) & 1);
+      same &= ((e >> b) & 1) ? bit : ~bit;
+    }
+    if (e >= 0) {
+      const int rank = popc_below_lane(same);
+      const int start = running[e];
+      __builtin_amdgcn_wave_barrier();
+      if (rank == 0) running[e] = start + __popcll(same);
+      const int row = start + rank;
+      scatter_index[i] = row;
+      if (gather_index) gather_index[row] = i / topk;
+      if (topk_index) topk_index[row] = i % topk;
+    } else {
+      __builtin_amdgcn_wave_barrier();
+      if (i < npairs) scatter_index[i] = -1;
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
 __global__ __launch_bounds__(kThreads) void route_scatter_kernel(
     const int32_t *__restrict__ choosed, int32_t npairs, int32_t topk, int32_t nexperts,
     int32_t nchunks, int32_t idbits, const int32_t *__restrict__ base,
@@ -104,35 +161,78 @@ __global__ __launch_bounds__(kThreads) void route_scatter_kernel(
     running[e] = s_off[e] + base[static_cast<size_t>(chunk) * nexperts + e];
   __builtin_amdgcn_wave_barrier();
 
-  const int first = chunk * kChunk;
-  for (int s = 0; s < kChunk / 64; ++s) {
-    const int i = first + s * 64 + lane;
-    int32_t e = -1;
-    if (i < npairs) {
-      e = choosed[i];
-      if (e < 0 || e >= nexperts) e = -1;
-    }
-    // Lanes that hold the same expert id as this lane.
-    uint64_t same = __ballot(e >= 0);
-    for (int b = 0; b < idbits; ++b) {
-      const uint64_t bit = __ballot((e >> b) & 1);
-      same &= ((e >> b) & 1) ? bit : ~bit;
-    }
-    if (e >= 0) {
-      const int rank = popc_below_lane(same);
-      const int start = running[e];
-      __builtin_amdgcn_wave_barrier();
-      if (rank == 0) running[e] = start + __popcll(same);
-      const int row = start + rank;
-      scatter_index[i] = row;
-      if (gather_index) gather_index[row] = i / topk;
-      if (topk_index) topk_index[row] = i % topk;
-    } else {
-      __builtin_amdgcn_wave_barrier();
-      if (i < npairs) scatter_index[i] = -1;
-    }
-    __builtin_amdgcn_wave_barrier();
+  scatter_range<false>(choosed, nullptr, chunk * kChunk, kChunk / 64, npairs, topk, nexperts, idbits, running,
+                       scatter_index, gather_index, topk_index);
+}
+
+// Whole sort in one launch for small inputs: one workgroup of 16 waves, wave w owns the contiguous pair
+// range [w*span, (w+1)*span).  The expert ids are first copied into LDS as 16-bit values by all 1024
+// lanes at once (one coalesced sweep; out-of-range ids become 0xffff), so that the two ordered passes
+// never wait on global memory.  LDS: hist[16][E] (becomes the per-wave running offsets), tot[E], off[E],
+// ids[npairs].
+constexpr int kSingleWaves = 16;
+constexpr int kSingleMaxPairs = 4096;  // beyond this the scattered index stores of one CU become the limit
+constexpr int kSingleMaxExperts = 512;
+
+__global__ __launch_bounds__(kSingleWaves * 64) void route_sort_single_kernel(
+    const int32_t *__restrict__ choosed, int32_t npairs, int32_t topk, int32_t nexperts, int32_t idbits,
+    int32_t *__restrict__ splits_out, int32_t *__restrict__ offsets_out, int32_t *__restrict__ scatter_index,
+    int32_t *__restrict__ gather_index, int32_t *__restrict__ topk_index) {
+  extern __shared__ int32_t s_mem[];
+  int32_t *s_hist = s_mem;                              // [kSingleWaves][nexperts]
+  int32_t *s_tot = s_mem + kSingleWaves * nexperts;     // [nexperts]
+  int32_t *s_off = s_tot + nexperts;                    // [nexperts]
+  uint16_t *s_ids = reinterpret_cast<uint16_t *>(s_off + nexperts);  // [npairs]
+  for (int i = threadIdx.x; i < npairs; i += blockDim.x) {
+    const int32_t e = choosed[i];
+    s_ids[i] = (e >= 0 && e < nexperts) ? static_cast<uint16_t>(e) : static_cast<uint16_t>(0xffff);
   }
+  const int wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int steps = ((npairs + kSingleWaves - 1) / kSingleWaves + 63) / 64;  // wave-steps per wave
+  const int first = wave * steps * 64;
+  for (int i = threadIdx.x; i < kSingleWaves * nexperts; i += blockDim.x) s_hist[i] = 0;
+  __syncthreads();
+  int32_t *my = s_hist + wave * nexperts;
+  for (int s = 0; s < steps; ++s) {
+    const int i = first + s * 64 + lane;
+    if (i < npairs) {
+      const int32_t e = s_ids[i];
+      if (e < nexperts) atomicAdd(&my[e], 1);
+    }
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < nexperts; e += blockDim.x) {
+    int run = 0;
+#pragma unroll
+    for (int w = 0; w < kSingleWaves; ++w) {
+      const int t = s_hist[w * nexperts + e];
+      s_hist[w * nexperts + e] = run;
+      run += t;
+    }
+    s_tot[e] = run;
+    if (splits_out) splits_out[e] = run;
+  }
+  __syncthreads();
+  if (wave == 0) {
+    int carry = 0;
+    for (int e0 = 0; e0 < nexperts; e0 += 64) {
+      const int e = e0 + lane;
+      const int v = e < nexperts ? s_tot[e] : 0;
+      const int incl = wave_inclusive_scan(v);
+      if (e < nexperts) {
+        s_off[e] = carry + incl - v;
+        if (offsets_out) offsets_out[e] = carry + incl - v;
+      }
+      carry += __shfl(incl, 63, 64);
+    }
+    if (lane == 0 && offsets_out) offsets_out[nexperts] = carry;
+  }
+  __syncthreads();
+  for (int e = lane; e < nexperts; e += 64) my[e] += s_off[e];
+  __builtin_amdgcn_wave_barrier();
+  scatter_range<true>(choosed, s_ids, first, steps, npairs, topk, nexperts, idbits, my, scatter_index,
+                      gather_index, topk_index);
 }
 
 __global__ __launch_bounds__(256) void gather_index_kernel(const int32_t *__restrict__ scatter_index,
@@ -188,6 +288,19 @@ extern "C" int fluxmi_moe_route_sort(const int32_t *choosed, int32_t ntokens, in
   int idbits = 0;
   while ((1 << idbits) < nexperts) ++idbits;
 
+  if (npairs <= kSingleMaxPairs && nexperts <= kSingleMaxExperts) {
+    static bool lds_attr_set = false;
+    if (!lds_attr_set) {
+      FLUXMI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(route_sort_single_kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024));
+      lds_attr_set = true;
+    }
+    hipLaunchKernelGGL(route_sort_single_kernel, dim3(1), dim3(kSingleWaves * 64),
+                       (kSingleWaves + 2) * nexperts * sizeof(int32_t) + ((npairs + 1) & ~1) * sizeof(uint16_t), s, choosed, npairs, topk, nexperts, idbits,
+                       splits, offsets, scatter_index, gather_index, topk_index);
+    FLUXMI_HIP_CHECK(hipGetLastError());
+    return FLUXMI_OK;
+  }
   const unsigned nblocks = static_cast<unsigned>((nchunks + kWavesPerBlock - 1) / kWavesPerBlock);
   if (nchunks > 0) {
     hipLaunchKernelGGL(route_hist_kernel, dim3(nblocks), dim3(kThreads),
