@@ -17,24 +17,31 @@
 // (those with equal blockIdx % 8) take a run of consecutive tiles; tiles of an expert are ordered
 // column-major (all row tiles of one weight panel first), so an XCD's L2 sees a few weight panels
 // shared by all row tiles of the expert.
+#include <cstdlib>
+
 #include "common.hpp"
 
 namespace fluxmi {
 namespace {
 
-constexpr int BM = 256;
-constexpr int BN = 256;
+constexpr int BM = 256;                    // rows of a macro tile
 constexpr int KBYTES = 64;                 // bytes of K per row per k-step
-#ifndef FLUXMI_GEMM_STAGES
-#define FLUXMI_GEMM_STAGES 5
-#endif
-#ifndef FLUXMI_GEMM_ISSUE_FIRST
-#define FLUXMI_GEMM_ISSUE_FIRST 0
-#endif
-constexpr int STAGES = FLUXMI_GEMM_STAGES;  // 5 x 32 KiB = the whole 160 KiB LDS of a CU
-constexpr int DIST = STAGES - 1;           // prefetch distance in k-steps
-constexpr int TILE_BYTES = 256 * KBYTES;   // one operand tile of one stage: 16 KiB
-constexpr int STAGE_BYTES = 2 * TILE_BYTES;
+constexpr int X_TILE_BYTES = BM * KBYTES;  // activation tile of one stage: 16 KiB
+
+// Two macro tile widths.  NBMAX = number of 32-column MFMA blocks per wave (4 waves across):
+//   NBMAX = 2: 256 x 256, stage 32 KiB, 5 stages;  NBMAX = 3: 256 x 384, stage 40 KiB, 4 stages.
+// Both fill the 160 KiB LDS of a CU.  The wide tile moves 17 % fewer operand bytes per FLOP through
+// L2, which is what bounds this kernel; its 192 accumulator registers leave room for the fragments of
+// only half a k-step, so it runs its memory / MFMA phases per 32-byte half step (KSPLIT = 2).
+template <int NBMAX>
+struct TileCfg {
+  static constexpr int BN = 128 * NBMAX;
+  static constexpr int W_TILE_BYTES = BN * KBYTES;
+  static constexpr int STAGE_BYTES = X_TILE_BYTES + W_TILE_BYTES;
+  static constexpr int STAGES = NBMAX == 2 ? 5 : 4;
+  static constexpr int DIST = STAGES - 1;  // prefetch distance in k-steps
+  static constexpr int KSPLIT = NBMAX == 2 ? 1 : 2;
+};
 constexpr int NTHREADS = 512;
 constexpr int kMaxExperts = 1024;
 
@@ -88,6 +95,12 @@ __device__ __forceinline__ f32x16 mfma_step<2>(const i32x4 (&w)[2], const i32x4 
   return acc;
 }
 
+// bf16 only: one 16-element half of a k-step.
+__device__ __forceinline__ f32x16 mfma_half_bf16(const i32x4 &w, const i32x4 &x, f32x16 acc) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, w), __builtin_bit_cast(bf16x8, x), acc,
+                                                 0, 0, 0);
+}
+
 template <>
 __device__ __forceinline__ f32x16 mfma_step<1>(const i32x4 (&w)[2], const i32x4 (&x)[2], f32x16 acc) {
   i32x8 wa, xa;
@@ -123,17 +136,22 @@ struct TileCtx {
 };
 
 // One output tile of (64*MB) rows x (128*NB) columns: MB x NB MFMA blocks of 32x32 per wave, waves laid
-// out 2 (rows) x 4 (columns).  (MB, NB) = (4, 2) is the 256x256 macro tile; (4, 1), (2, 2) and (2, 1) are
-// the 256x128, 128x256 and 128x128 pieces a tile of the last, partly filled round is cut into.
-template <int ELT, int MB, int NB>
+// out 2 (rows) x 4 (columns).  (MB, NB) = (4, NBMAX) is the macro tile; (4, 1) and (2, 1) are the 256x128
+// and 128x128 pieces a tile of the last, partly filled round is cut into.  KSPLIT = 2 runs the
+// memory / MFMA phase pair once per half k-step with half the fragment registers (bf16 only).
+template <int ELT, int NBMAX, int MB, int NB, int KSPLIT>
 __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, TileCtx &c, int e,
                                           int row_base, int rows_e, int m0, int n0) {
+  using Cfg = TileCfg<NBMAX>;
+  constexpr int STAGES = Cfg::STAGES, DIST = Cfg::DIST, STAGE_BYTES = Cfg::STAGE_BYTES;
   constexpr int XLOADS = MB / 2;             // direct-to-LDS instructions per wave per stage, X tile
   constexpr int WLOADS = NB;                 // same, W tile
   constexpr int LOADS = XLOADS + WLOADS;
+  constexpr int NS = 2 / KSPLIT;             // 16-byte fragment chunks read per phase
+  static_assert(KSPLIT == 1 || ELT == 2, "half k-steps exist for bf16 only");
   const int wave = c.wave, lane = c.lane, wm = c.wm, wn = c.wn, nk = c.nk;
   const int x_frag_base = wm * (32 * MB) * KBYTES;
-  const int w_frag_base = TILE_BYTES + wn * (32 * NB) * KBYTES;
+  const int w_frag_base = X_TILE_BYTES + wn * (32 * NB) * KBYTES;
 
   // Global source pointers of this lane's fill instructions (k offset added per step).  Instruction q
   // of a tile covers rows [16q, 16q+16); tail rows re-read the last valid row.
@@ -165,7 +183,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, Ti
     for (int j = 0; j < XLOADS; ++j) load_to_lds16(xsrc[j] + koff, stage + (XLOADS * wave + j) * 1024);
 #pragma unroll
     for (int j = 0; j < WLOADS; ++j)
-      load_to_lds16(wsrc[j] + koff, stage + TILE_BYTES + (WLOADS * wave + j) * 1024);
+      load_to_lds16(wsrc[j] + koff, stage + X_TILE_BYTES + (WLOADS * wave + j) * 1024);
   };
 
   f32x16 acc[MB][NB];
@@ -190,40 +208,52 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, Ti
   if (wm == 1) __builtin_amdgcn_s_barrier();  // group 1 runs one phase behind group 0
 
   for (int ks = 0; ks < nk; ++ks) {
-    // ---- memory phase ---------------------------------------------------------------------------
     const uint8_t *stage = smem + c.read_stage * STAGE_BYTES;
     c.read_stage = c.read_stage + 1 == STAGES ? 0 : c.read_stage + 1;
     const bool more = ks + DIST < nk;
-    i32x4 xf[MB][2], wf[NB][2];
 #pragma unroll
-    for (int j = 0; j < NB; ++j)
+    for (int sub = 0; sub < KSPLIT; ++sub) {
+      // ---- memory phase -------------------------------------------------------------------------
+      i32x4 xf[MB][NS], wf[NB][NS];
 #pragma unroll
-      for (int s = 0; s < 2; ++s)
-        wf[j][s] = *reinterpret_cast<const i32x4 *>(stage + w_frag_base + j * 32 * KBYTES + c.frag_off[s]);
+      for (int j = 0; j < NB; ++j)
 #pragma unroll
-    for (int i = 0; i < MB; ++i)
+        for (int s = 0; s < NS; ++s)
+          wf[j][s] = *reinterpret_cast<const i32x4 *>(stage + w_frag_base + j * 32 * KBYTES +
+                                                      c.frag_off[KSPLIT == 1 ? s : sub]);
 #pragma unroll
-      for (int s = 0; s < 2; ++s)
-        xf[i][s] = *reinterpret_cast<const i32x4 *>(stage + x_frag_base + i * 32 * KBYTES + c.frag_off[s]);
-    if (more) {
-      issue_stage(ks + DIST);
-      FLUXMI_WAITCNT((DIST - 1) * LOADS, 0);  // stage ks+1 landed, fragments in registers
-    } else {
-      FLUXMI_WAITCNT(0, 0);
+      for (int i = 0; i < MB; ++i)
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+          xf[i][s] = *reinterpret_cast<const i32x4 *>(stage + x_frag_base + i * 32 * KBYTES +
+                                                      c.frag_off[KSPLIT == 1 ? s : sub]);
+      if (sub == 0 && more) issue_stage(ks + DIST);
+      if (sub == KSPLIT - 1) {
+        if (more) {
+          FLUXMI_WAITCNT((DIST - 1) * LOADS, 0);  // stage ks+1 landed, fragments in registers
+        } else {
+          FLUXMI_WAITCNT(0, 0);
+        }
+      } else {
+        FLUXMI_WAITCNT(63, 0);  // fragments in registers; global loads keep flying
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      // ---- compute phase ------------------------------------------------------------------------
+      __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+      for (int i = 0; i < MB; ++i)
+#pragma unroll
+        for (int j = 0; j < NB; ++j) {
+          if constexpr (KSPLIT == 1) acc[i][j] = mfma_step<ELT>(wf[j], xf[i], acc[i][j]);
+          else acc[i][j] = mfma_half_bf16(wf[j][0], xf[i][0], acc[i][j]);
+        }
+      __builtin_amdgcn_s_setprio(0);
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
     }
-    __builtin_amdgcn_sched_barrier(0);
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_sched_barrier(0);
-    // ---- compute phase --------------------------------------------------------------------------
-    __builtin_amdgcn_s_setprio(1);
-#pragma unroll
-    for (int i = 0; i < MB; ++i)
-#pragma unroll
-      for (int j = 0; j < NB; ++j) acc[i][j] = mfma_step<ELT>(wf[j], xf[i], acc[i][j]);
-    __builtin_amdgcn_s_setprio(0);
-    __builtin_amdgcn_sched_barrier(0);
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_sched_barrier(0);
   }
   if (wm == 0) __builtin_amdgcn_s_barrier();  // re-align the two groups
 
@@ -272,8 +302,10 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, Ti
   }
 }
 
-template <int ELT>
+template <int ELT, int NBMAX>
 __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmParams p) {
+  constexpr int BN = TileCfg<NBMAX>::BN;
+  constexpr int KSPLIT = TileCfg<NBMAX>::KSPLIT;
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];  // STAGES x (X tile | W tile)
 
   TileCtx c;
@@ -332,12 +364,12 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
     }
     total_tiles = __builtin_amdgcn_readfirstlane(acc_tiles);
   }
-  // Full rounds run whole 256x256 tiles.  The tiles of the last, partly filled round are cut into
-  // `pieces` parts (4: 128x128, 2: 256x128) when that still fits one round, so that the chip does not
-  // idle while a fraction of the CUs finishes whole tiles.
+  // Full rounds run whole macro tiles.  The tiles of the last, partly filled round are cut into
+  // `pieces` parts (NBMAX pieces of 256x128, or 2*NBMAX of 128x128) when that still fits one round, so
+  // that the chip does not idle while a fraction of the CUs finishes whole tiles.
   const int full_items = (total_tiles / grid) * grid;
   const int rem_tiles = total_tiles - full_items;
-  const int pieces = rem_tiles * 4 <= grid ? 4 : (rem_tiles * 2 <= grid ? 2 : 1);
+  const int pieces = rem_tiles * 2 * NBMAX <= grid ? 2 * NBMAX : (rem_tiles * NBMAX <= grid ? NBMAX : 1);
   const int total_items = full_items + rem_tiles * pieces;
 
   // ---- schedule: walk the experts once, in step with this workgroup's increasing tile ids ----------
@@ -382,14 +414,14 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
     int n0 = nt * BN;
 
     if (item < full_items || pieces == 1) {
-      gemm_tile<ELT, 4, 2>(p, smem, c, e, row_base, rows_e, m0, n0);
-    } else if (pieces == 2) {
+      gemm_tile<ELT, NBMAX, 4, NBMAX, KSPLIT>(p, smem, c, e, row_base, rows_e, m0, n0);
+    } else if (pieces == NBMAX) {
       n0 += piece * 128;
-      if (n0 < p.n) gemm_tile<ELT, 4, 1>(p, smem, c, e, row_base, rows_e, m0, n0);
+      if (n0 < p.n) gemm_tile<ELT, NBMAX, 4, 1, 1>(p, smem, c, e, row_base, rows_e, m0, n0);
     } else {
-      m0 += (piece >> 1) * 128;
-      n0 += (piece & 1) * 128;
-      if (m0 < rows_e && n0 < p.n) gemm_tile<ELT, 2, 1>(p, smem, c, e, row_base, rows_e, m0, n0);
+      m0 += (piece / NBMAX) * 128;
+      n0 += (piece % NBMAX) * 128;
+      if (m0 < rows_e && n0 < p.n) gemm_tile<ELT, NBMAX, 2, 1, 1>(p, smem, c, e, row_base, rows_e, m0, n0);
     }
   }
 }
@@ -468,7 +500,35 @@ bool mfma_path_ok(const fluxmi_grouped_gemm_args *a) {
          (a->col_scale == nullptr || aligned16(a->col_scale));
 }
 
-size_t mfma_lds_bytes() { return static_cast<size_t>(STAGES) * STAGE_BYTES; }
+template <int NBMAX>
+constexpr size_t mfma_lds_bytes() {
+  return static_cast<size_t>(TileCfg<NBMAX>::STAGES) * TileCfg<NBMAX>::STAGE_BYTES;
+}
+
+// Macro tile width: 384 columns (bf16 only) unless padding N up to a multiple of 384 wastes clearly
+// more work than padding it to a multiple of 256.  FLUXMI_GEMM_TILE_N=256|384 overrides.
+int pick_nbmax(const fluxmi_grouped_gemm_args *a) {
+  if (a->dtype != FLUXMI_BF16) return 2;
+  if (const char *env = getenv("FLUXMI_GEMM_TILE_N")) {
+    if (atoi(env) == 256) return 2;
+    if (atoi(env) == 384) return 3;
+  }
+  const int64_t pad2 = (static_cast<int64_t>(a->n) + 255) / 256 * 256;
+  const int64_t pad3 = (static_cast<int64_t>(a->n) + 383) / 384 * 384;
+  return pad3 * 100 <= pad2 * 104 ? 3 : 2;
+}
+
+template <int ELT, int NBMAX>
+int launch_mfma(const GemmParams &p, int grid, hipStream_t s) {
+  static bool attr_set = false;
+  if (!attr_set) {
+    FLUXMI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(grouped_gemm_mfma_kernel<ELT, NBMAX>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+    attr_set = true;
+  }
+  hipLaunchKernelGGL((grouped_gemm_mfma_kernel<ELT, NBMAX>), dim3(grid), dim3(NTHREADS), mfma_lds_bytes<NBMAX>(), s, p);
+  return FLUXMI_OK;
+}
 
 }  // namespace
 }  // namespace fluxmi
@@ -517,28 +577,15 @@ extern "C" int fluxmi_grouped_gemm(const fluxmi_grouped_gemm_args *args, void *,
   FLUXMI_REQUIRE(cus > 0, FLUXMI_ERR_HIP, "grouped_gemm: cannot query the device");
 
   if (mfma_path_ok(args)) {
-    const size_t lds = mfma_lds_bytes();
+    const int nbmax = pick_nbmax(args);
     // Upper bound of the tile count: never launch more workgroups than tiles.
-    const int64_t tiles_n = (args->n + BN - 1) / BN;
+    const int64_t tiles_n = (args->n + 128 * nbmax - 1) / (128 * nbmax);
     const int64_t max_tiles = (static_cast<int64_t>(args->max_rows) / BM + args->nexperts) * tiles_n;
     const int grid = static_cast<int>(max_tiles < cus ? max_tiles : cus);
-    if (args->dtype == FLUXMI_BF16) {
-      static bool attr_set = false;
-      if (!attr_set) {
-        FLUXMI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(grouped_gemm_mfma_kernel<2>),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-        attr_set = true;
-      }
-      hipLaunchKernelGGL(grouped_gemm_mfma_kernel<2>, dim3(grid), dim3(NTHREADS), lds, s, p);
-    } else {
-      static bool attr_set = false;
-      if (!attr_set) {
-        FLUXMI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(grouped_gemm_mfma_kernel<1>),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-        attr_set = true;
-      }
-      hipLaunchKernelGGL(grouped_gemm_mfma_kernel<1>, dim3(grid), dim3(NTHREADS), lds, s, p);
-    }
+    int rc;
+    if (args->dtype == FLUXMI_BF16) rc = nbmax == 3 ? launch_mfma<2, 3>(p, grid, s) : launch_mfma<2, 2>(p, grid, s);
+    else rc = launch_mfma<1, 2>(p, grid, s);
+    if (rc != FLUXMI_OK) return rc;
   } else {
     const int grid = cus * 8;
     if (args->dtype == FLUXMI_BF16)
