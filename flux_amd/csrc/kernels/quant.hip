@@ -158,34 +158,50 @@ __global__ __launch_bounds__(256) void quant_row_long_kernel(const uint16_t *__r
 // ---- one scale per (row, 128-column block) -----------------------------------------------------
 // 16 consecutive lanes own one block (16 vectors of 8 elements); the amax reduction is four xor
 // shuffles inside that lane group.
+template <int THREADS_PER_ROW>
 __global__ __launch_bounds__(256) void quant_block128_kernel(const uint16_t *__restrict__ x,
                                                              int64_t rows, int32_t nvec,
                                                              int32_t nblocks, float eps,
                                                              uint8_t *__restrict__ q,
                                                              float *__restrict__ scale_inv,
                                                              int32_t permute) {
-  const int64_t gid = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-  const int64_t grp = gid >> 4;  // (row, block) pair
-  const int lane16 = static_cast<int>(gid & 15);
-  const int64_t row = grp / nblocks;
-  const int32_t blk = static_cast<int32_t>(grp - row * nblocks);
-  const int32_t c = blk * 16 + lane16;
-  const bool ok = row < rows && c < nvec;
-  u32x4 v = u32x4{0u, 0u, 0u, 0u};
-  if (ok) v = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x) + row * nvec + c);
-  uint32_t m = amax8(v);
+  // THREADS_PER_ROW lanes walk one row in steps of THREADS_PER_ROW vectors; blocks start at multiples
+  // of 16 vectors, so the 16 lanes of a block always step together.
+  constexpr int kRowsPerBlock = 256 / THREADS_PER_ROW;
+  const int tid = threadIdx.x % THREADS_PER_ROW;
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock + threadIdx.x / THREADS_PER_ROW;
+  if (row >= rows) return;
+  const u32x4 *src = reinterpret_cast<const u32x4 *>(x) + row * nvec;
+  u32x2 *dst = reinterpret_cast<u32x2 *>(q) + row * nvec;
+  for (int c = tid; c < nblocks * 16; c += THREADS_PER_ROW) {
+    const bool ok = c < nvec;  // a partial last block: missing vectors count as zeros
+    u32x4 v = u32x4{0u, 0u, 0u, 0u};
+    if (ok) v = __builtin_nontemporal_load(src + c);
+    uint32_t m = amax8(v);
 #pragma unroll
-  for (int off = 8; off > 0; off >>= 1) m = max(m, static_cast<uint32_t>(__shfl_xor(static_cast<int>(m), off, 64)));
-  const float scale = compute_scale(__uint_as_float(m), eps);
-  if (row < rows && lane16 == 0) {
-    const float inv = static_cast<float>(1.0 / static_cast<double>(scale));
-    if (permute)
-      scale_inv[(row >> 7) * (static_cast<int64_t>(nblocks) * 128) + static_cast<int64_t>(blk) * 128 +
-                (row & 127)] = inv;
-    else
-      scale_inv[row * nblocks + blk] = inv;
+    for (int off = 8; off > 0; off >>= 1)
+      m = max(m, static_cast<uint32_t>(__shfl_xor(static_cast<int>(m), off, 64)));
+    const float scale = compute_scale(__uint_as_float(m), eps);
+    if ((c & 15) == 0) {
+      const int blk = c >> 4;
+      const float inv = static_cast<float>(1.0 / static_cast<double>(scale));
+      if (permute)
+        scale_inv[(row >> 7) * (static_cast<int64_t>(nblocks) * 128) + static_cast<int64_t>(blk) * 128 +
+                  (row & 127)] = inv;
+      else
+        scale_inv[row * nblocks + blk] = inv;
+    }
+    if (ok) __builtin_nontemporal_store(cast8(v, scale), dst + c);
   }
-  if (ok) __builtin_nontemporal_store(cast8(v, scale), reinterpret_cast<u32x2 *>(q) + row * nvec + c);
+}
+
+template <int TPR>
+void launch_block128(hipStream_t s, const uint16_t *x, int64_t rows, int32_t nvec, int32_t nblocks, float eps,
+                     uint8_t *q, float *si, int32_t permute) {
+  constexpr int kRowsPerBlock = 256 / TPR;
+  const unsigned grid = static_cast<unsigned>((rows + kRowsPerBlock - 1) / kRowsPerBlock);
+  hipLaunchKernelGGL((quant_block128_kernel<TPR>), dim3(grid), dim3(256), 0, s, x, rows, nvec, nblocks, eps, q, si,
+                     permute);
 }
 
 template <int TPR, int VPT>
@@ -225,11 +241,11 @@ extern "C" int fluxmi_quant_e4m3_rowwise(const void *x_bf16, int64_t rows, int64
 
   if (block_cols == 128) {
     const int32_t nblocks = static_cast<int32_t>((cols + 127) / 128);
-    const int64_t lanes = rows * nblocks * 16;
-    const int64_t grid = (lanes + 255) / 256;
-    FLUXMI_REQUIRE(grid <= INT32_MAX, FLUXMI_ERR_UNSUPPORTED, "quant_e4m3_rowwise: matrix too large");
-    hipLaunchKernelGGL(quant_block128_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, s, x,
-                       rows, nvec, nblocks, eps, q, scale_inv_out, permute_scale);
+    FLUXMI_REQUIRE(rows <= INT32_MAX, FLUXMI_ERR_UNSUPPORTED, "quant_e4m3_rowwise: too many rows");
+    const int32_t lanes = nblocks * 16;
+    if (lanes <= 64) launch_block128<64>(s, x, rows, nvec, nblocks, eps, q, scale_inv_out, permute_scale);
+    else if (lanes <= 128) launch_block128<128>(s, x, rows, nvec, nblocks, eps, q, scale_inv_out, permute_scale);
+    else launch_block128<256>(s, x, rows, nvec, nblocks, eps, q, scale_inv_out, permute_scale);
   } else {
     FLUXMI_REQUIRE(rows <= INT32_MAX, FLUXMI_ERR_UNSUPPORTED, "quant_e4m3_rowwise: too many rows");
     if (nvec <= 64) launch_row<64, 1>(s, x, rows, nvec, eps, q, scale_inv_out);
