@@ -26,7 +26,7 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per grouped-GEMM launch on C3 (mean of layer0 and layer1): FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000
 # from the two rocprofv3 --pmc runs summarised in profiles/bench_c3_pmc_counters.md (scale factors from the
 # 1 GiB copy of --calib-copy).  Only valid for the C3 workload with the fp32 layer1 intermediate.
-GEMM_TRAFFIC_C3_BYTES = 3.897e9
+GEMM_TRAFFIC_C3_BYTES = 3.653e9
 
 
 def parse():
@@ -181,6 +181,20 @@ def main():
             kernels[f"quant_e4m3_{rows}x{cols}"] = {"ms": round(t_q, 4), "gbs": round(b_q / t_q * 1e-6, 1),
                                                     "frac_hbm": round(b_q / t_q * 1e-6 / PEAK_HBM_GBS, 4)}
         del zb
+        # fp8 grouped GEMM at the C5 shape (one GPU's expert share: E=32, M=32768, K=2048, N=7168), row x column
+        # scales and top-8 weight in the epilogue.
+        e5, m5, k5, n5 = 32, 32768, 2048, 7168
+        a8 = torch.randn(m5, k5, generator=gen, device=dev).to(torch.float8_e4m3fn)
+        b8 = (torch.randn(e5, n5, k5, generator=gen, device=dev)).to(torch.float8_e4m3fn)
+        sp5 = torch.full((e5,), m5 // e5, dtype=torch.int32, device=dev)
+        rs5 = torch.rand(m5, generator=gen, device=dev)
+        cs5 = torch.rand(e5, n5, generator=gen, device=dev)
+        d5 = torch.empty(m5, n5, dtype=torch.bfloat16, device=dev)
+        t_f8 = time_loop(torch, lambda: capi.grouped_gemm(a8, b8, sp5, out=d5, row_scale=rs5, col_scale=cs5), 20)
+        f_f8 = 2.0 * m5 * k5 * n5
+        kernels["gemm_fp8_c5_layer1"] = {"ms": round(t_f8, 4), "tflops": round(f_f8 / t_f8 * 1e-9, 1),
+                                         "frac_fp8_peak": round(f_f8 / t_f8 * 1e-9 / PEAK_FP8_TFLOPS, 4)}
+        del a8, b8, d5
 
     if a.calib_copy:
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
