@@ -21,12 +21,13 @@ extern "C" const char *fluxmi_last_error(void) { return fluxmi::g_last_error; }
 extern "C" int fluxmi_device_cu_count(void) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return -1;
-  static int cached_dev = -1;
-  static int cached_cus = 0;
-  if (dev == cached_dev) return cached_cus;
+  static std::atomic<int> cached[64];  // CU count per device id, 0 = not queried yet
+  if (dev >= 0 && dev < 64) {
+    const int c = cached[dev].load(std::memory_order_relaxed);
+    if (c > 0) return c;
+  }
   int cus = 0;
   if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return -1;
-  cached_dev = dev;
-  cached_cus = cus;
+  if (dev >= 0 && dev < 64) cached[dev].store(cus, std::memory_order_relaxed);
   return cus;
 }

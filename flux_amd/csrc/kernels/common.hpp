@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 
@@ -31,6 +32,19 @@ void set_error(const char *fmt, ...);
     }                                                                                     \
   } while (0)
 
+// Raises the dynamic-LDS limit of `kernel` to `bytes` once per device (the attribute lives with the
+// device's copy of the code object).  `done_mask` is a function-local static of the caller, one bit per
+// device id; a lost race only repeats the idempotent call.
+inline int ensure_dynamic_lds(const void *kernel, int bytes, std::atomic<uint64_t> &done_mask) {
+  int dev = 0;
+  FLUXMI_HIP_CHECK(hipGetDevice(&dev));
+  const uint64_t bit = uint64_t{1} << (dev & 63);
+  if (done_mask.load(std::memory_order_acquire) & bit) return FLUXMI_OK;
+  FLUXMI_HIP_CHECK(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
+  done_mask.fetch_or(bit, std::memory_order_release);
+  return FLUXMI_OK;
+}
+
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 constexpr int kWave = 64;
@@ -44,12 +58,6 @@ __device__ __forceinline__ int lane_id() {
 __device__ __forceinline__ int popc_below_lane(uint64_t mask) {
   return __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(mask >> 32),
                                    __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(mask), 0u));
-}
-
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
-  return v;
 }
 
 // Inclusive prefix sum across the 64 lanes of a wave.

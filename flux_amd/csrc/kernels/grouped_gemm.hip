@@ -520,12 +520,10 @@ int pick_nbmax(const fluxmi_grouped_gemm_args *a) {
 
 template <int ELT, int NBMAX>
 int launch_mfma(const GemmParams &p, int grid, hipStream_t s) {
-  static bool attr_set = false;
-  if (!attr_set) {
-    FLUXMI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(grouped_gemm_mfma_kernel<ELT, NBMAX>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_done{0};
+  const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(grouped_gemm_mfma_kernel<ELT, NBMAX>), 160 * 1024,
+                                    lds_done);
+  if (rc != FLUXMI_OK) return rc;
   hipLaunchKernelGGL((grouped_gemm_mfma_kernel<ELT, NBMAX>), dim3(grid), dim3(NTHREADS), mfma_lds_bytes<NBMAX>(), s, p);
   return FLUXMI_OK;
 }

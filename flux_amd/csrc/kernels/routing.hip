@@ -289,12 +289,9 @@ extern "C" int fluxmi_moe_route_sort(const int32_t *choosed, int32_t ntokens, in
   while ((1 << idbits) < nexperts) ++idbits;
 
   if (npairs <= kSingleMaxPairs && nexperts <= kSingleMaxExperts) {
-    static bool lds_attr_set = false;
-    if (!lds_attr_set) {
-      FLUXMI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(route_sort_single_kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024));
-      lds_attr_set = true;
-    }
+    static std::atomic<uint64_t> lds_done{0};
+    const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(route_sort_single_kernel), 128 * 1024, lds_done);
+    if (rc != FLUXMI_OK) return rc;
     hipLaunchKernelGGL(route_sort_single_kernel, dim3(1), dim3(kSingleWaves * 64),
                        (kSingleWaves + 2) * nexperts * sizeof(int32_t) + ((npairs + 1) & ~1) * sizeof(uint16_t), s, choosed, npairs, topk, nexperts, idbits,
                        splits, offsets, scatter_index, gather_index, topk_index);
