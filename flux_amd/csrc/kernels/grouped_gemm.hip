@@ -1,22 +1,30 @@
 // Grouped GEMM over ragged per-expert row counts: D[r,:] = scale(r,:) * A[gather(r),:] @ B[e(r)]^T.
 //
-// Persistent kernel, one 512-thread workgroup (8 waves, 2 per SIMD) per CU, macro tile 256 rows x 256
+// Persistent kernel, one 256-thread workgroup (4 waves, one per SIMD) per CU, macro tile 256 rows x 256
 // columns, k-step of 64 bytes per row (32 bf16 or 64 fp8).  Both operand tiles are staged in LDS by
-// direct-to-LDS global loads (no register staging) in a 5-deep ring; the row gather of A is folded into
-// the per-lane global address of those loads.  Each wave owns a 128x64 slice of the macro tile
-// (4x2 MFMA blocks of 32x32, fp32 accumulators).  The two waves that share a SIMD run one phase apart
-// ("ping-pong"): while one issues its LDS fragment reads and the next global loads, the other issues
-// MFMAs, and workgroup barriers keep them alternating.
+// direct-to-LDS global loads (no register staging) in a ring of five 32 KiB stages; the row gather of A
+// is folded into the per-lane global address of those loads.  Each wave owns a 128 x 128 quarter of the
+// macro tile (4x4 MFMA blocks of 32x32, 256 fp32 accumulator registers) and runs a software pipeline
+// of its own: while the MFMAs of k-step s run on one set of fragment registers, the fragments of step
+// s+1 are read from LDS into a second set and the ring fills of steps s+4 / s+5 are issued, all in a
+// fixed interleaving (one fragment read per MFMA over the first half of the step, one fill every
+// fourth MFMA).  One workgroup barrier per k-step publishes the landed stage.
+//
+// Ring fills are issued in pairs of k-steps: the two 64-byte halves of a 128-byte line are requested
+// back to back (they go to different stages), so the second request hits the line the first one
+// brought into the vector L1 and L2 sees one request per line instead of two.
 //
 // The MFMA "A" operand is the weight fragment and the "B" operand the activation fragment, i.e. the
 // hardware computes D^T blocks: a lane then holds, for one output row, four consecutive output columns
-// per accumulator quad, which makes the epilogue's stores 8-byte packed bf16x4.
+// per accumulator quad.  The epilogue passes each 64-row x 32-column block through a wave-private LDS
+// window in fp32 and reads it back with eight lanes per row, so that one store instruction writes 64
+// (bf16) or 128 (fp32) contiguous bytes of each row.
 //
 // Tile schedule: every wave walks the device-resident `splits` with scalar loads, in step with the
 // increasing logical tile ids of its workgroup; ids are assigned so that the workgroups of one XCD
-// (those with equal blockIdx % 8) take a run of consecutive tiles; tiles of an expert are ordered
-// column-major (all row tiles of one weight panel first), so an XCD's L2 sees a few weight panels
-// shared by all row tiles of the expert.
+// (those with equal blockIdx % 8) take a run of consecutive tiles; tiles of an expert are ordered in
+// groups of at most 8 row tiles, each group walked column-major over the weight panels, so an XCD's L2
+// sees a few weight panels shared by the row tiles of a group.
 #include <cstdlib>
 
 #include "common.hpp"
@@ -25,30 +33,22 @@ namespace fluxmi {
 namespace {
 
 constexpr int BM = 256;                    // rows of a macro tile
+constexpr int BN = 256;                    // columns of a macro tile
 constexpr int KBYTES = 64;                 // bytes of K per row per k-step
 constexpr int X_TILE_BYTES = BM * KBYTES;  // activation tile of one stage: 16 KiB
-
-// Two macro tile widths.  NBMAX = number of 32-column MFMA blocks per wave (4 waves across):
-//   NBMAX = 2: 256 x 256, stage 32 KiB, 5 stages;  NBMAX = 3: 256 x 384, stage 40 KiB, 4 stages.
-// Both fill the 160 KiB LDS of a CU.  The wide tile moves 17 % fewer operand bytes per FLOP through
-// L2, which is what bounds this kernel; its 192 accumulator registers leave room for the fragments of
-// only half a k-step, so it runs its memory / MFMA phases per 32-byte half step (KSPLIT = 2).
-template <int NBMAX>
-struct TileCfg {
-  static constexpr int BN = 128 * NBMAX;
-  static constexpr int W_TILE_BYTES = BN * KBYTES;
-  static constexpr int STAGE_BYTES = X_TILE_BYTES + W_TILE_BYTES;
-  static constexpr int STAGES = NBMAX == 2 ? 5 : 4;
-  static constexpr int DIST = STAGES - 1;  // prefetch distance in k-steps
-  static constexpr int KSPLIT = NBMAX == 2 ? 1 : 2;
-};
-constexpr int NTHREADS = 512;
+constexpr int W_TILE_BYTES = BN * KBYTES;
+constexpr int STAGE_BYTES = X_TILE_BYTES + W_TILE_BYTES;
+constexpr int STAGES = 5;                  // 160 KiB: the whole LDS of a CU
+constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
+constexpr int NTHREADS = 256;
 constexpr int kMaxExperts = 1024;
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef int i32x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 struct GemmParams {
@@ -83,36 +83,37 @@ __device__ __forceinline__ void load_to_lds16(const uint8_t *src, uint8_t *lds_b
   __builtin_amdgcn_global_load_lds((gbl_ptr_t)src, (lds_ptr_t)lds_base, 16, 0, 0);
 }
 
-template <int ELT>
-__device__ __forceinline__ f32x16 mfma_step(const i32x4 (&w)[2], const i32x4 (&x)[2], f32x16 acc);
-
-template <>
-__device__ __forceinline__ f32x16 mfma_step<2>(const i32x4 (&w)[2], const i32x4 (&x)[2], f32x16 acc) {
-  acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, w[0]),
-                                                __builtin_bit_cast(bf16x8, x[0]), acc, 0, 0, 0);
-  acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, w[1]),
-                                                __builtin_bit_cast(bf16x8, x[1]), acc, 0, 0, 0);
-  return acc;
+// Two floats to packed bf16, round to nearest even (one v_cvt_pk_bf16_f32).
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  const f32x2 v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
 }
 
-// bf16 only: one 16-element half of a k-step.
-__device__ __forceinline__ f32x16 mfma_half_bf16(const i32x4 &w, const i32x4 &x, f32x16 acc) {
-  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, w), __builtin_bit_cast(bf16x8, x), acc,
-                                                 0, 0, 0);
-}
+// Source of the fills of a k-step past the end of K (odd number of k-steps): both operands read zeros.
+__device__ __attribute__((aligned(1024))) const uint8_t g_zero_page[1024] = {};
 
-template <>
-__device__ __forceinline__ f32x16 mfma_step<1>(const i32x4 (&w)[2], const i32x4 (&x)[2], f32x16 acc) {
-  i32x8 wa, xa;
+// MFMA number t of a k-step.  bf16: 2 * MB * NB instructions of 32x32x16, the two 16-element halves of
+// the step one after the other.  fp8: MB * NB instructions of 32x32x64 (both 16-byte chunks at once).
+template <int ELT, int MB, int NB>
+__device__ __forceinline__ void mfma_slot(int t, const i32x4 (&xf)[MB][2], const i32x4 (&wf)[NB][2],
+                                          f32x16 (&acc)[MB][NB]) {
+  if constexpr (ELT == 2) {
+    const int s = t / (MB * NB), i = (t % (MB * NB)) / NB, j = t % NB;
+    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, wf[j][s]),
+                                                        __builtin_bit_cast(bf16x8, xf[i][s]), acc[i][j], 0, 0, 0);
+  } else {
+    const int i = t / NB, j = t % NB;
+    i32x8 wa, xa;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    wa[i] = w[0][i];
-    wa[4 + i] = w[1][i];
-    xa[i] = x[0][i];
-    xa[4 + i] = x[1][i];
+    for (int v = 0; v < 4; ++v) {
+      wa[v] = wf[j][0][v];
+      wa[4 + v] = wf[j][1][v];
+      xa[v] = xf[i][0][v];
+      xa[4 + v] = xf[i][1][v];
+    }
+    // cbsz = blgp = 0: both operands e4m3; zero scale operands select the unscaled form (scale 1).
+    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wa, xa, acc[i][j], 0, 0, 0, 0, 0, 0);
   }
-  // cbsz = blgp = 0: both operands e4m3; zero scale operands select the unscaled form (scale 1).
-  return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wa, xa, acc, 0, 0, 0, 0, 0, 0);
 }
 
 // Clamped row count of expert e: negative entries count as 0 and rows past max_rows do not exist.
@@ -123,32 +124,98 @@ __device__ __forceinline__ int expert_rows(const GemmParams &p, int e, int row_b
   return rows;
 }
 
-// Per-lane constants and ring state shared by all tile shapes.
+// Per-lane constants shared by all tile shapes.
 struct TileCtx {
   int wave, lane, wn, wm;
   int fill_row, fill_chunk;
   int frag_off[2];
-  int fill_stage;  // ring slot the next issued k-step goes to
-  int read_stage;  // ring slot of the k-step read next
   int nk;
   int64_t kbytes;
   float scalar;
 };
 
-// One output tile of (64*MB) rows x (128*NB) columns: MB x NB MFMA blocks of 32x32 per wave, waves laid
-// out 2 (rows) x 4 (columns).  (MB, NB) = (4, NBMAX) is the macro tile; (4, 1) and (2, 1) are the 256x128
-// and 128x128 pieces a tile of the last, partly filled round is cut into.  KSPLIT = 2 runs the
-// memory / MFMA phase pair once per half k-step with half the fragment registers (bf16 only).
-template <int ELT, int NBMAX, int MB, int NB, int KSPLIT>
-__device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, TileCtx &c, int e,
-                                          int row_base, int rows_e, int m0, int n0) {
-  using Cfg = TileCfg<NBMAX>;
-  constexpr int STAGES = Cfg::STAGES, DIST = Cfg::DIST, STAGE_BYTES = Cfg::STAGE_BYTES;
-  constexpr int XLOADS = MB / 2;             // direct-to-LDS instructions per wave per stage, X tile
-  constexpr int WLOADS = NB;                 // same, W tile
+// Epilogue of one wave: acc (32*MB rows x 32*NB columns, MFMA layout) -> scaled, cast, stored.
+// FULL: every row and column of the wave's quarter exists and rows are stored where they are (no
+// scatter), so no store is predicated.  OUT_F32 selects the output element type.
+template <int MB, int NB, bool FULL, bool OUT_F32>
+__device__ __forceinline__ void store_tile(const GemmParams &p, uint8_t *window, const TileCtx &c, int e, int row_base,
+                                           int rows_e, int wrow0, int wcol0, const f32x16 (&acc)[MB][NB]) {
+  static_assert(MB % 2 == 0, "the window holds two 32-row blocks");
+  const int lane = c.lane;
+  const int h = lane >> 5;
+  const float tile_scale = c.scalar * (p.alpha ? p.alpha[e] : 1.f);
+  float rs[MB];
+#pragma unroll
+  for (int i = 0; i < MB; ++i) {
+    const int m = wrow0 + i * 32 + (lane & 31);
+    rs[i] = tile_scale * ((p.row_scale && (FULL || m < rows_e)) ? p.row_scale[row_base + m] : 1.f);
+  }
+  const int rr0 = lane >> 3;  // row of this lane within a group of 8 rows (store phase)
+  const int cc = lane & 7;    // its 4-column chunk
+#pragma unroll
+  for (int j = 0; j < NB; ++j) {
+    const int col = wcol0 + j * 32 + cc * 4;
+    float4 cs = make_float4(1.f, 1.f, 1.f, 1.f);
+    if (p.col_scale && (FULL || col < p.n))
+      cs = *reinterpret_cast<const float4 *>(p.col_scale + static_cast<int64_t>(e) * p.n + col);
+#pragma unroll
+    for (int ip = 0; ip < MB / 2; ++ip) {
+      // write phase: lane holds row (ii*32 + lane%32), columns q*8 + h*4 .. +3 = 16-byte chunk 2q+h
+#pragma unroll
+      for (int ii = 0; ii < 2; ++ii) {
+        const int i = ip * 2 + ii;
+        const int r = ii * 32 + (lane & 31);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const float4 v = make_float4(acc[i][j][4 * q + 0] * rs[i], acc[i][j][4 * q + 1] * rs[i],
+                                       acc[i][j][4 * q + 2] * rs[i], acc[i][j][4 * q + 3] * rs[i]);
+          *reinterpret_cast<float4 *>(window + r * 128 + (((2 * q + h) ^ ((r >> 1) & 7)) << 4)) = v;
+        }
+      }
+      // store phase: 8 lanes per row, 8 rows per instruction
+      float4 v[8];
+#pragma unroll
+      for (int it = 0; it < 8; ++it) {
+        const int rr = it * 8 + rr0;
+        v[it] = *reinterpret_cast<const float4 *>(window + rr * 128 + ((cc ^ ((rr >> 1) & 7)) << 4));
+      }
+#pragma unroll
+      for (int it = 0; it < 8; ++it) {
+        const int m = wrow0 + ip * 64 + it * 8 + rr0;
+        int64_t drow = row_base + m;
+        if constexpr (!FULL) {
+          if (m >= rows_e || col >= p.n) continue;  // n % 4 == 0: a chunk is all in or all out
+          if (p.scatter_d) {
+            drow = p.scatter_d[row_base + m];
+            if (drow < 0 || drow >= p.max_rows) continue;
+          }
+        }
+        const float4 o = make_float4(v[it].x * cs.x, v[it].y * cs.y, v[it].z * cs.z, v[it].w * cs.w);
+        if constexpr (OUT_F32) {
+          *reinterpret_cast<float4 *>(static_cast<float *>(p.d) + drow * p.n + col) = o;
+        } else {
+          u32x2 b;
+          b[0] = pack_bf16x2(o.x, o.y);
+          b[1] = pack_bf16x2(o.z, o.w);
+          *reinterpret_cast<u32x2 *>(static_cast<uint16_t *>(p.d) + drow * p.n + col) = b;
+        }
+      }
+    }
+  }
+}
+
+// One output tile of (64*MB) rows x (64*NB) columns at rows [m0, ..) of expert e, columns [n0, ..).
+// (MB, NB) = (4, 4) is the macro tile; (4, 2) and (2, 2) are the 256x128 and 128x128 pieces a tile of
+// the last, partly filled round is cut into.  Waves are laid out 2 x 2.
+template <int ELT, int MB, int NB>
+__device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, const TileCtx &c, int e, int row_base,
+                                          int rows_e, int m0, int n0) {
+  constexpr int XLOADS = MB;           // direct-to-LDS instructions per wave per stage, X tile
+  constexpr int WLOADS = NB;           // same, W tile
   constexpr int LOADS = XLOADS + WLOADS;
-  constexpr int NS = 2 / KSPLIT;             // 16-byte fragment chunks read per phase
-  static_assert(KSPLIT == 1 || ELT == 2, "half k-steps exist for bf16 only");
+  constexpr int NR = LOADS * 2;        // fragment reads per k-step
+  constexpr int NM = MB * NB * (ELT == 2 ? 2 : 1);  // MFMAs per k-step
+  constexpr int RSPAN = NM / 2;        // MFMA slots over which the fragment reads of a step are spread
   const int wave = c.wave, lane = c.lane, wm = c.wm, wn = c.wn, nk = c.nk;
   const int x_frag_base = wm * (32 * MB) * KBYTES;
   const int w_frag_base = X_TILE_BYTES + wn * (32 * NB) * KBYTES;
@@ -174,16 +241,17 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, Ti
     if (wr > p.n - 1) wr = p.n - 1;
     wsrc[j] = p.b + (static_cast<int64_t>(e) * p.n + wr) * c.kbytes + c.fill_chunk * 16;
   }
+  const uint8_t *zsrc = g_zero_page + lane * 16;
 
-  auto issue_stage = [&](int kstep) {
-    uint8_t *stage = smem + c.fill_stage * STAGE_BYTES;
-    c.fill_stage = c.fill_stage + 1 == STAGES ? 0 : c.fill_stage + 1;
-    const int64_t koff = static_cast<int64_t>(kstep) * KBYTES;
-#pragma unroll
-    for (int j = 0; j < XLOADS; ++j) load_to_lds16(xsrc[j] + koff, stage + (XLOADS * wave + j) * 1024);
-#pragma unroll
-    for (int j = 0; j < WLOADS; ++j)
-      load_to_lds16(wsrc[j] + koff, stage + X_TILE_BYTES + (WLOADS * wave + j) * 1024);
+  // Fill instruction q (X rows first, then W rows) of k-step `kstep` into ring slot `slot`.  A k-step
+  // past the end of K is clamped to the last one (never consumed) or, if it is the phantom second half
+  // of the last pair of an odd K, filled with zeros.
+  auto fill_one = [&](int slot, int kstep, int q) {
+    uint8_t *stage = smem + slot * STAGE_BYTES;
+    const bool zero = kstep == nk;
+    const int64_t koff = static_cast<int64_t>(kstep < nk ? kstep : nk - 1) * KBYTES;
+    if (q < XLOADS) load_to_lds16(zero ? zsrc : xsrc[q] + koff, stage + (XLOADS * wave + q) * 1024);
+    else load_to_lds16(zero ? zsrc : wsrc[q - XLOADS] + koff, stage + X_TILE_BYTES + (WLOADS * wave + (q - XLOADS)) * 1024);
   };
 
   f32x16 acc[MB][NB];
@@ -194,126 +262,111 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, Ti
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-  // ---- prologue: fill DIST stages ---------------------------------------------------------------
+  i32x4 xa[MB][2], wa[NB][2], xb[MB][2], wb[NB][2];
+  // Fragment read r of a k-step: chunk s = r / LOADS of W block q (q < NB) or X block q - NB.
+  auto read_one = [&](const uint8_t *stage, int r, i32x4 (&xf)[MB][2], i32x4 (&wf)[NB][2]) {
+    const int s = r / LOADS, q = r % LOADS;
+    if (q < NB) wf[q][s] = *reinterpret_cast<const i32x4 *>(stage + w_frag_base + q * 32 * KBYTES + c.frag_off[s]);
+    else xf[q - NB][s] = *reinterpret_cast<const i32x4 *>(stage + x_frag_base + (q - NB) * 32 * KBYTES + c.frag_off[s]);
+  };
+
+  // Ring slots: k-step s lives in slot s % 5.  `rslot` is the slot of the step whose fragments are read
+  // next, `fslot` the slot the next requested step goes to.
+  int rslot = 0, fslot = 0;
+  auto next_slot = [](int s) { return s + 1 == STAGES ? 0 : s + 1; };
+
+  // One k-step `ks`: MFMAs on `cur` (read during the previous step), fragments of step ks+1 into `nxt`,
+  // and half of the fills of the pair of steps (e+4, e+5), e = ks rounded down to even: that pair is
+  // requested over the two steps e and e+1, X/W row group by row group, both k-steps of a row group
+  // back to back.
+  int pslot0 = 0, pslot1 = 0;
+  auto step = [&](int ks, bool even, i32x4 (&xc)[MB][2], i32x4 (&wc)[NB][2], i32x4 (&xn)[MB][2], i32x4 (&wn_)[NB][2]) {
+    // Stage ks+1 has landed once the pair it belongs to is complete; fills are counted in issue order.
+    if (even) {
+      FLUXMI_WAITCNT(2 * LOADS, 15);  // all but the pair requested during steps ks-2, ks-1
+    } else {
+      FLUXMI_WAITCNT(LOADS, 15);      // all but the half pair requested during step ks-1
+    }
+    __builtin_amdgcn_s_barrier();     // ... for every wave's share; and everybody is done reading stage ks
+    __builtin_amdgcn_sched_barrier(0);
+    const uint8_t *rstage = smem + rslot * STAGE_BYTES;
+    rslot = next_slot(rslot);
+    if (even) {
+      pslot0 = fslot;
+      pslot1 = next_slot(fslot);
+      fslot = next_slot(pslot1);
+    }
+    const int e0 = even ? ks : ks - 1;
+#pragma unroll
+    for (int t = 0; t < NM; ++t) {
+#pragma unroll
+      for (int r = 0; r < NR; ++r)
+        if (r * RSPAN / NR == t) read_one(rstage, r, xn, wn_);
+#pragma unroll
+      for (int d = 0; d < 2 * LOADS; ++d)
+        if ((d * (2 * NM) / (2 * LOADS) + 1) % (2 * NM) == t + (even ? 0 : NM))
+          fill_one((d & 1) ? pslot1 : pslot0, e0 + 4 + (d & 1), d >> 1);
+      mfma_slot<ELT, MB, NB>(t, xc, wc, acc);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    FLUXMI_WAITCNT(63, 0);  // the fragments of the next step are in registers (requested long ago)
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  // ---- prologue: request k-steps 0..3 as two pairs, wait for the first pair ------------------------
   FLUXMI_WAITCNT(0, 0);  // stores of the previous tile's epilogue
 #pragma unroll
-  for (int s = 0; s < DIST; ++s)
-    if (s < nk) issue_stage(s);
-  if (nk >= DIST) {
-    FLUXMI_WAITCNT((DIST - 1) * LOADS, 15);
-  } else {
-    FLUXMI_WAITCNT(0, 15);
+  for (int s = 0; s < 4; s += 2) {
+    const int s0 = fslot, s1 = next_slot(fslot);
+    fslot = next_slot(s1);
+#pragma unroll
+    for (int q = 0; q < LOADS; ++q) {
+      fill_one(s0, s, q);
+      fill_one(s1, s + 1, q);
+    }
   }
+  FLUXMI_WAITCNT(2 * LOADS, 15);
   __builtin_amdgcn_s_barrier();
-  if (wm == 1) __builtin_amdgcn_s_barrier();  // group 1 runs one phase behind group 0
-
-  for (int ks = 0; ks < nk; ++ks) {
-    const uint8_t *stage = smem + c.read_stage * STAGE_BYTES;
-    c.read_stage = c.read_stage + 1 == STAGES ? 0 : c.read_stage + 1;
-    const bool more = ks + DIST < nk;
+  {
+    const uint8_t *stage = smem + rslot * STAGE_BYTES;
+    rslot = next_slot(rslot);
 #pragma unroll
-    for (int sub = 0; sub < KSPLIT; ++sub) {
-      // ---- memory phase -------------------------------------------------------------------------
-      i32x4 xf[MB][NS], wf[NB][NS];
-#pragma unroll
-      for (int j = 0; j < NB; ++j)
-#pragma unroll
-        for (int s = 0; s < NS; ++s)
-          wf[j][s] = *reinterpret_cast<const i32x4 *>(stage + w_frag_base + j * 32 * KBYTES +
-                                                      c.frag_off[KSPLIT == 1 ? s : sub]);
-#pragma unroll
-      for (int i = 0; i < MB; ++i)
-#pragma unroll
-        for (int s = 0; s < NS; ++s)
-          xf[i][s] = *reinterpret_cast<const i32x4 *>(stage + x_frag_base + i * 32 * KBYTES +
-                                                      c.frag_off[KSPLIT == 1 ? s : sub]);
-      if (sub == 0 && more) issue_stage(ks + DIST);
-      if (sub == KSPLIT - 1) {
-        if (more) {
-          FLUXMI_WAITCNT((DIST - 1) * LOADS, 0);  // stage ks+1 landed, fragments in registers
-        } else {
-          FLUXMI_WAITCNT(0, 0);
-        }
-      } else {
-        FLUXMI_WAITCNT(63, 0);  // fragments in registers; global loads keep flying
-      }
-      __builtin_amdgcn_sched_barrier(0);
-      __builtin_amdgcn_s_barrier();
-      __builtin_amdgcn_sched_barrier(0);
-      // ---- compute phase ------------------------------------------------------------------------
-      __builtin_amdgcn_s_setprio(1);
-#pragma unroll
-      for (int i = 0; i < MB; ++i)
-#pragma unroll
-        for (int j = 0; j < NB; ++j) {
-          if constexpr (KSPLIT == 1) acc[i][j] = mfma_step<ELT>(wf[j], xf[i], acc[i][j]);
-          else acc[i][j] = mfma_half_bf16(wf[j][0], xf[i][0], acc[i][j]);
-        }
-      __builtin_amdgcn_s_setprio(0);
-      __builtin_amdgcn_sched_barrier(0);
-      __builtin_amdgcn_s_barrier();
-      __builtin_amdgcn_sched_barrier(0);
-    }
+    for (int r = 0; r < NR; ++r) read_one(stage, r, xa, wa);
   }
-  if (wm == 0) __builtin_amdgcn_s_barrier();  // re-align the two groups
-
-  // ---- epilogue: scale, cast, packed stores -------------------------------------------------------
-  const float tile_scale = c.scalar * (p.alpha ? p.alpha[e] : 1.f);
-#pragma unroll
-  for (int i = 0; i < MB; ++i) {
-    const int m = m0 + wm * (32 * MB) + i * 32 + (lane & 31);
-    if (m >= rows_e) continue;
-    const int64_t srow = row_base + m;
-    const float rs = tile_scale * (p.row_scale ? p.row_scale[srow] : 1.f);
-    int64_t drow = srow;
-    if (p.scatter_d) {
-      drow = p.scatter_d[srow];
-      if (drow < 0 || drow >= p.max_rows) continue;
-    }
-    uint16_t *dptr = static_cast<uint16_t *>(p.d) + drow * p.n;
-    float *dptr32 = static_cast<float *>(p.d) + drow * p.n;
-#pragma unroll
-    for (int j = 0; j < NB; ++j) {
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int n = n0 + wn * (32 * NB) + j * 32 + q * 8 + (lane >> 5) * 4;
-        if (n >= p.n) continue;  // n % 4 == 0 is required, so a quad is all in or all out
-        float v0 = acc[i][j][4 * q + 0] * rs;
-        float v1 = acc[i][j][4 * q + 1] * rs;
-        float v2 = acc[i][j][4 * q + 2] * rs;
-        float v3 = acc[i][j][4 * q + 3] * rs;
-        if (p.col_scale) {
-          const float4 cs = *reinterpret_cast<const float4 *>(p.col_scale + static_cast<int64_t>(e) * p.n + n);
-          v0 *= cs.x;
-          v1 *= cs.y;
-          v2 *= cs.z;
-          v3 *= cs.w;
-        }
-        if (p.d_fp32) {
-          *reinterpret_cast<float4 *>(dptr32 + n) = make_float4(v0, v1, v2, v3);
-        } else {
-          u32x2 o;
-          o[0] = float_to_bf16_bits(v0) | (static_cast<uint32_t>(float_to_bf16_bits(v1)) << 16);
-          o[1] = float_to_bf16_bits(v2) | (static_cast<uint32_t>(float_to_bf16_bits(v3)) << 16);
-          *reinterpret_cast<u32x2 *>(dptr + n) = o;
-        }
-      }
-    }
+  FLUXMI_WAITCNT(63, 0);  // in registers before the first step's barrier lets anyone refill that slot
+  // An odd number of k-steps runs one phantom step on zero fragments.
+  for (int ks = 0; ks < nk; ks += 2) {
+    step(ks, true, xa, wa, xb, wb);
+    step(ks + 1, false, xb, wb, xa, wa);
   }
+
+  // ---- epilogue ---------------------------------------------------------------------------------
+  FLUXMI_WAITCNT(0, 0);          // this wave's trailing ring fills have landed
+  __builtin_amdgcn_s_barrier();  // ... and everybody else's; nobody reads the ring any more
+  uint8_t *window = smem + wave * 8192;
+  const int wrow0 = m0 + wm * (32 * MB);
+  const int wcol0 = n0 + wn * (32 * NB);
+  const bool full = wrow0 + 32 * MB <= rows_e && wcol0 + 32 * NB <= p.n && p.scatter_d == nullptr;
+  if (full) {
+    if (p.d_fp32) store_tile<MB, NB, true, true>(p, window, c, e, row_base, rows_e, wrow0, wcol0, acc);
+    else store_tile<MB, NB, true, false>(p, window, c, e, row_base, rows_e, wrow0, wcol0, acc);
+  } else {
+    if (p.d_fp32) store_tile<MB, NB, false, true>(p, window, c, e, row_base, rows_e, wrow0, wcol0, acc);
+    else store_tile<MB, NB, false, false>(p, window, c, e, row_base, rows_e, wrow0, wcol0, acc);
+  }
+  __builtin_amdgcn_s_barrier();  // the LDS windows are free again before the next tile's fills start
 }
 
-template <int ELT, int NBMAX>
+template <int ELT>
 __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmParams p) {
-  constexpr int BN = TileCfg<NBMAX>::BN;
-  constexpr int KSPLIT = TileCfg<NBMAX>::KSPLIT;
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];  // STAGES x (X tile | W tile)
 
   TileCtx c;
   const int tid = threadIdx.x;
   c.wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: branches on it stay uniform
   c.lane = tid & 63;
-  c.wn = c.wave & 3;   // column slice
-  c.wm = c.wave >> 2;  // row slice == ping-pong group
+  c.wn = c.wave & 1;   // column half
+  c.wm = c.wave >> 1;  // row half
   const int lane = c.lane;
   const int tiles_n = (p.n + BN - 1) / BN;
   c.kbytes = static_cast<int64_t>(p.k) * ELT;
@@ -336,8 +389,6 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
   }
   c.scalar = p.scalar;
   if (p.scalar_dev) c.scalar *= p.scalar_dev[0];
-  c.fill_stage = 0;
-  c.read_stage = 0;
 
   const int grid = gridDim.x;
   const int bid = blockIdx.x;
@@ -365,11 +416,11 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
     total_tiles = __builtin_amdgcn_readfirstlane(acc_tiles);
   }
   // Full rounds run whole macro tiles.  The tiles of the last, partly filled round are cut into
-  // `pieces` parts (NBMAX pieces of 256x128, or 2*NBMAX of 128x128) when that still fits one round, so
-  // that the chip does not idle while a fraction of the CUs finishes whole tiles.
+  // `pieces` parts (2 pieces of 256x128, or 4 of 128x128) when that still fits one round, so that the
+  // chip does not idle while a fraction of the CUs finishes whole tiles.
   const int full_items = (total_tiles / grid) * grid;
   const int rem_tiles = total_tiles - full_items;
-  const int pieces = rem_tiles * 2 * NBMAX <= grid ? 2 * NBMAX : (rem_tiles * NBMAX <= grid ? NBMAX : 1);
+  const int pieces = rem_tiles * 4 <= grid ? 4 : (rem_tiles * 2 <= grid ? 2 : 1);
   const int total_items = full_items + rem_tiles * pieces;
 
   // ---- schedule: walk the experts once, in step with this workgroup's increasing tile ids ----------
@@ -414,14 +465,14 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
     int n0 = nt * BN;
 
     if (item < full_items || pieces == 1) {
-      gemm_tile<ELT, NBMAX, 4, NBMAX, KSPLIT>(p, smem, c, e, row_base, rows_e, m0, n0);
-    } else if (pieces == NBMAX) {
+      gemm_tile<ELT, 4, 4>(p, smem, c, e, row_base, rows_e, m0, n0);
+    } else if (pieces == 2) {
       n0 += piece * 128;
-      if (n0 < p.n) gemm_tile<ELT, NBMAX, 4, 1, 1>(p, smem, c, e, row_base, rows_e, m0, n0);
+      if (n0 < p.n) gemm_tile<ELT, 4, 2>(p, smem, c, e, row_base, rows_e, m0, n0);
     } else {
-      m0 += (piece / NBMAX) * 128;
-      n0 += (piece % NBMAX) * 128;
-      if (m0 < rows_e && n0 < p.n) gemm_tile<ELT, NBMAX, 2, 1, 1>(p, smem, c, e, row_base, rows_e, m0, n0);
+      m0 += (piece >> 1) * 128;
+      n0 += (piece & 1) * 128;
+      if (m0 < rows_e && n0 < p.n) gemm_tile<ELT, 2, 2>(p, smem, c, e, row_base, rows_e, m0, n0);
     }
   }
 }
@@ -500,31 +551,12 @@ bool mfma_path_ok(const fluxmi_grouped_gemm_args *a) {
          (a->col_scale == nullptr || aligned16(a->col_scale));
 }
 
-template <int NBMAX>
-constexpr size_t mfma_lds_bytes() {
-  return static_cast<size_t>(TileCfg<NBMAX>::STAGES) * TileCfg<NBMAX>::STAGE_BYTES;
-}
-
-// Macro tile width: 384 columns (bf16 only) unless padding N up to a multiple of 384 wastes clearly
-// more work than padding it to a multiple of 256.  FLUXMI_GEMM_TILE_N=256|384 overrides.
-int pick_nbmax(const fluxmi_grouped_gemm_args *a) {
-  if (a->dtype != FLUXMI_BF16) return 2;
-  if (const char *env = getenv("FLUXMI_GEMM_TILE_N")) {
-    if (atoi(env) == 256) return 2;
-    if (atoi(env) == 384) return 3;
-  }
-  const int64_t pad2 = (static_cast<int64_t>(a->n) + 255) / 256 * 256;
-  const int64_t pad3 = (static_cast<int64_t>(a->n) + 383) / 384 * 384;
-  return pad3 * 100 <= pad2 * 104 ? 3 : 2;
-}
-
-template <int ELT, int NBMAX>
+template <int ELT>
 int launch_mfma(const GemmParams &p, int grid, hipStream_t s) {
   static std::atomic<uint64_t> lds_done{0};
-  const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(grouped_gemm_mfma_kernel<ELT, NBMAX>), 160 * 1024,
-                                    lds_done);
+  const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(grouped_gemm_mfma_kernel<ELT>), LDS_BYTES, lds_done);
   if (rc != FLUXMI_OK) return rc;
-  hipLaunchKernelGGL((grouped_gemm_mfma_kernel<ELT, NBMAX>), dim3(grid), dim3(NTHREADS), mfma_lds_bytes<NBMAX>(), s, p);
+  hipLaunchKernelGGL((grouped_gemm_mfma_kernel<ELT>), dim3(grid), dim3(NTHREADS), LDS_BYTES, s, p);
   return FLUXMI_OK;
 }
 
@@ -575,14 +607,11 @@ extern "C" int fluxmi_grouped_gemm(const fluxmi_grouped_gemm_args *args, void *,
   FLUXMI_REQUIRE(cus > 0, FLUXMI_ERR_HIP, "grouped_gemm: cannot query the device");
 
   if (mfma_path_ok(args)) {
-    const int nbmax = pick_nbmax(args);
     // Upper bound of the tile count: never launch more workgroups than tiles.
-    const int64_t tiles_n = (args->n + 128 * nbmax - 1) / (128 * nbmax);
+    const int64_t tiles_n = (args->n + BN - 1) / BN;
     const int64_t max_tiles = (static_cast<int64_t>(args->max_rows) / BM + args->nexperts) * tiles_n;
     const int grid = static_cast<int>(max_tiles < cus ? max_tiles : cus);
-    int rc;
-    if (args->dtype == FLUXMI_BF16) rc = nbmax == 3 ? launch_mfma<2, 3>(p, grid, s) : launch_mfma<2, 2>(p, grid, s);
-    else rc = launch_mfma<1, 2>(p, grid, s);
+    const int rc = args->dtype == FLUXMI_BF16 ? launch_mfma<2>(p, grid, s) : launch_mfma<1>(p, grid, s);
     if (rc != FLUXMI_OK) return rc;
   } else {
     const int grid = cus * 8;
