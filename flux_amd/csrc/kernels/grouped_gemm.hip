@@ -26,6 +26,7 @@
 // groups of at most 8 row tiles, each group walked column-major over the weight panels, so an XCD's L2
 // sees a few weight panels shared by the row tiles of a group.
 #include <cstdlib>
+#include <type_traits>
 
 #include "common.hpp"
 
@@ -89,7 +90,7 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
 }
 
-// Source of the fills of a k-step past the end of K (odd number of k-steps): both operands read zeros.
+// Source of the ring fills of a k-step past the end of K: every lane reads 16 zero bytes.
 __device__ __attribute__((aligned(1024))) const uint8_t g_zero_page[1024] = {};
 
 // MFMA number t of a k-step.  bf16: 2 * MB * NB instructions of 32x32x16, the two 16-element halves of
@@ -204,6 +205,21 @@ __device__ __forceinline__ void store_tile(const GemmParams &p, uint8_t *window,
   }
 }
 
+// Compile-time loop: f(integral_constant<int, I>) for I in [0, N).
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F &&f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<I + 1, N>(f);
+  }
+}
+
+// Buffer resource over [base, base + bytes): loads past the end return zero instead of faulting.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const uint8_t *base, int64_t bytes) {
+  const uint32_t n = bytes > 0xffffffffll ? 0xffffffffu : static_cast<uint32_t>(bytes < 0 ? 0 : bytes);
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(base), 0, static_cast<int>(n), 0x00020000);
+}
+
 // One output tile of (64*MB) rows x (64*NB) columns at rows [m0, ..) of expert e, columns [n0, ..).
 // (MB, NB) = (4, 4) is the macro tile; (4, 2) and (2, 2) are the 256x128 and 128x128 pieces a tile of
 // the last, partly filled round is cut into.  Waves are laid out 2 x 2.
@@ -217,41 +233,61 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
   constexpr int NM = MB * NB * (ELT == 2 ? 2 : 1);  // MFMAs per k-step
   constexpr int RSPAN = NM / 2;        // MFMA slots over which the fragment reads of a step are spread
   const int wave = c.wave, lane = c.lane, wm = c.wm, wn = c.wn, nk = c.nk;
-  const int x_frag_base = wm * (32 * MB) * KBYTES;
-  const int w_frag_base = X_TILE_BYTES + wn * (32 * NB) * KBYTES;
 
-  // Global source pointers of this lane's fill instructions (k offset added per step).  Instruction q
-  // of a tile covers rows [16q, 16q+16); tail rows re-read the last valid row.
-  const uint8_t *xsrc[XLOADS];
-  const uint8_t *wsrc[WLOADS];
+  // Ring fills address global memory through buffer resources: a scalar base per operand, a
+  // loop-invariant 32-bit byte offset per lane and fill instruction, and the k offset as scalar offset
+  // plus immediate.  Fill instruction q of a tile covers rows [16q, 16q+16); tail rows re-read the last
+  // valid row.
+  const bool gathered = p.gather_a != nullptr;
+  const uint8_t *xbase = gathered ? p.a : p.a + static_cast<int64_t>(row_base + m0) * c.kbytes;
+  const int64_t xrows = gathered ? p.a_rows : rows_e - m0;
+  const int64_t xbytes = xrows > 0 ? xrows * c.kbytes : 0xffffffffll;
+  const uint8_t *wbase = p.b + (static_cast<int64_t>(e) * p.n + n0) * c.kbytes;
+  const int64_t wbytes = static_cast<int64_t>(p.n - n0) * c.kbytes;
+  // The loop runs whole trips of ten k-steps, the surplus ones on zero fragments: a k-step past the end
+  // of K is filled from a page of zeros (every lane at offset 16 * lane).  `in_k[h]` says whether the
+  // h-th k-step of the pair being requested exists.
+  const __amdgpu_buffer_rsrc_t xrsrc = make_rsrc(xbase, xbytes);
+  const __amdgpu_buffer_rsrc_t wrsrc = make_rsrc(wbase, wbytes);
+  const __amdgpu_buffer_rsrc_t zrsrc = make_rsrc(g_zero_page, 1024);
+  const uint32_t zoff = lane * 16;
+  const int kbytes32 = static_cast<int>(c.kbytes);  // K * element size fits 31 bits (K itself is an int32)
+  bool in_k[2] = {true, true};
+  uint32_t xoff[XLOADS], woff[WLOADS];
 #pragma unroll
   for (int j = 0; j < XLOADS; ++j) {
     int xr = m0 + (XLOADS * wave + j) * 16 + c.fill_row;
     if (xr > rows_e - 1) xr = rows_e - 1;
-    int64_t arow = row_base + xr;
-    if (p.gather_a) {
-      arow = p.gather_a[arow];
+    int64_t arow = xr - m0;
+    if (gathered) {
+      arow = p.gather_a[row_base + xr];
       if (p.a_rows > 0) arow = arow < 0 ? 0 : (arow >= p.a_rows ? p.a_rows - 1 : arow);
     }
-    xsrc[j] = p.a + arow * c.kbytes + c.fill_chunk * 16;
+    xoff[j] = static_cast<uint32_t>(arow * c.kbytes) + c.fill_chunk * 16;
   }
 #pragma unroll
   for (int j = 0; j < WLOADS; ++j) {
     int wr = n0 + (WLOADS * wave + j) * 16 + c.fill_row;
     if (wr > p.n - 1) wr = p.n - 1;
-    wsrc[j] = p.b + (static_cast<int64_t>(e) * p.n + wr) * c.kbytes + c.fill_chunk * 16;
+    woff[j] = static_cast<uint32_t>((wr - n0) * c.kbytes) + c.fill_chunk * 16;
   }
-  const uint8_t *zsrc = g_zero_page + lane * 16;
+  // LDS destinations of this wave's fill instructions inside a stage (X rows first, then W rows).
+  uint8_t *xdst = smem + (XLOADS * wave) * 1024;
+  uint8_t *wdst = smem + X_TILE_BYTES + (WLOADS * wave) * 1024;
 
-  // Fill instruction q (X rows first, then W rows) of k-step `kstep` into ring slot `slot`.  A k-step
-  // past the end of K is clamped to the last one (never consumed) or, if it is the phantom second half
-  // of the last pair of an odd K, filled with zeros.
-  auto fill_one = [&](int slot, int kstep, int q) {
-    uint8_t *stage = smem + slot * STAGE_BYTES;
-    const bool zero = kstep == nk;
-    const int64_t koff = static_cast<int64_t>(kstep < nk ? kstep : nk - 1) * KBYTES;
-    if (q < XLOADS) load_to_lds16(zero ? zsrc : xsrc[q] + koff, stage + (XLOADS * wave + q) * 1024);
-    else load_to_lds16(zero ? zsrc : wsrc[q - XLOADS] + koff, stage + X_TILE_BYTES + (WLOADS * wave + (q - XLOADS)) * 1024);
+  // Fill instruction Q of the k-step at byte offset kbase + KOFF of every row (the H-th of its pair), into
+  // ring slot SLOT.  The k offset travels as the scalar offset: an instruction immediate would also be
+  // added to the LDS address.
+  auto fill_one = [&](auto CHECK, auto SLOT, auto Q, auto H, int kbase, auto KOFF) {
+    constexpr int slot = decltype(SLOT)::value, q = decltype(Q)::value, koff = decltype(KOFF)::value;
+    constexpr int h = decltype(H)::value;
+    const bool in = !decltype(CHECK)::value || in_k[h];  // unchecked: the caller knows the k-step exists
+    if constexpr (q < XLOADS)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(in ? xrsrc : zrsrc, (lds_ptr_t)(xdst + slot * STAGE_BYTES + q * 1024), 16,
+                                               static_cast<int>(in ? xoff[q] : zoff), in ? kbase + koff : 0, 0, 0);
+    else
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(in ? wrsrc : zrsrc, (lds_ptr_t)(wdst + slot * STAGE_BYTES + (q - XLOADS) * 1024),
+                                               16, static_cast<int>(in ? woff[q - XLOADS] : zoff), in ? kbase + koff : 0, 0, 0);
   };
 
   f32x16 acc[MB][NB];
@@ -262,82 +298,111 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
+  // Fragment addresses: per lane and 16-byte chunk s a base for each operand; a stage and block add a
+  // compile-time offset.  LDS instructions carry 16 bits of offset, so three bases 64 KiB apart.
+  const uint8_t *xfrag[3][2], *wfrag[3][2];
+#pragma unroll
+  for (int hi = 0; hi < 3; ++hi)
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      xfrag[hi][s] = smem + hi * 65536 + wm * (32 * MB) * KBYTES + c.frag_off[s];
+      wfrag[hi][s] = smem + hi * 65536 + X_TILE_BYTES + wn * (32 * NB) * KBYTES + c.frag_off[s];
+    }
   i32x4 xa[MB][2], wa[NB][2], xb[MB][2], wb[NB][2];
-  // Fragment read r of a k-step: chunk s = r / LOADS of W block q (q < NB) or X block q - NB.
-  auto read_one = [&](const uint8_t *stage, int r, i32x4 (&xf)[MB][2], i32x4 (&wf)[NB][2]) {
-    const int s = r / LOADS, q = r % LOADS;
-    if (q < NB) wf[q][s] = *reinterpret_cast<const i32x4 *>(stage + w_frag_base + q * 32 * KBYTES + c.frag_off[s]);
-    else xf[q - NB][s] = *reinterpret_cast<const i32x4 *>(stage + x_frag_base + (q - NB) * 32 * KBYTES + c.frag_off[s]);
+  // Fragment read R of the k-step in ring slot SLOT: chunk s = R / LOADS of W block q (q < NB) or of
+  // X block q - NB.
+  auto read_one = [&](auto SLOT, auto R, i32x4 (&xf)[MB][2], i32x4 (&wf)[NB][2]) {
+    constexpr int slot = decltype(SLOT)::value, r = decltype(R)::value;
+    constexpr int s = r / LOADS, q = r % LOADS;
+    constexpr int hi = (slot * STAGE_BYTES) / 65536, lo = (slot * STAGE_BYTES) % 65536;
+    if constexpr (q < NB) wf[q][s] = *reinterpret_cast<const i32x4 *>(wfrag[hi][s] + lo + q * 32 * KBYTES);
+    else xf[q - NB][s] = *reinterpret_cast<const i32x4 *>(xfrag[hi][s] + lo + (q - NB) * 32 * KBYTES);
   };
 
-  // Ring slots: k-step s lives in slot s % 5.  `rslot` is the slot of the step whose fragments are read
-  // next, `fslot` the slot the next requested step goes to.
-  int rslot = 0, fslot = 0;
-  auto next_slot = [](int s) { return s + 1 == STAGES ? 0 : s + 1; };
-
-  // One k-step `ks`: MFMAs on `cur` (read during the previous step), fragments of step ks+1 into `nxt`,
-  // and half of the fills of the pair of steps (e+4, e+5), e = ks rounded down to even: that pair is
-  // requested over the two steps e and e+1, X/W row group by row group, both k-steps of a row group
-  // back to back.
-  int pslot0 = 0, pslot1 = 0;
-  auto step = [&](int ks, bool even, i32x4 (&xc)[MB][2], i32x4 (&wc)[NB][2], i32x4 (&xn)[MB][2], i32x4 (&wn_)[NB][2]) {
-    // Stage ks+1 has landed once the pair it belongs to is complete; fills are counted in issue order.
-    if (even) {
-      FLUXMI_WAITCNT(2 * LOADS, 15);  // all but the pair requested during steps ks-2, ks-1
+  // One k-step, number U within a run of ten (ring of five slots x two fragment sets: after ten steps
+  // every slot index and register role repeats, so all of them are compile-time constants here).
+  // MFMAs run on `cur` (read during the previous step), the fragments of the next step go into `nxt`,
+  // and half of the fills of the pair of steps (E+4, E+5), E = U rounded down to even, are issued:
+  // that pair is requested over the two steps E and E+1, row group by row group, both k-steps of a row
+  // group back to back (the second one hits the line the first one brought into L1).
+  auto step = [&](auto CHECK, auto U, int kbase, i32x4 (&xc)[MB][2], i32x4 (&wc)[NB][2], i32x4 (&xn)[MB][2], i32x4 (&wn_)[NB][2]) {
+    constexpr int u = decltype(U)::value;
+    constexpr bool even = (u & 1) == 0;
+    constexpr int e0 = u & ~1;
+    // Stage u+1 has landed once the pair it belongs to is complete; fills are counted in issue order.
+    if constexpr (even) {
+      FLUXMI_WAITCNT(2 * LOADS, 15);  // all but the pair requested during the last two steps
     } else {
-      FLUXMI_WAITCNT(LOADS, 15);      // all but the half pair requested during step ks-1
+      FLUXMI_WAITCNT(LOADS, 15);      // all but the half pair requested during the last step
     }
-    __builtin_amdgcn_s_barrier();     // ... for every wave's share; and everybody is done reading stage ks
+    __builtin_amdgcn_s_barrier();     // ... for every wave's share; and everybody is done reading stage u
     __builtin_amdgcn_sched_barrier(0);
-    const uint8_t *rstage = smem + rslot * STAGE_BYTES;
-    rslot = next_slot(rslot);
-    if (even) {
-      pslot0 = fslot;
-      pslot1 = next_slot(fslot);
-      fslot = next_slot(pslot1);
+    if constexpr (even && decltype(CHECK)::value) {
+      in_k[0] = kbase + (e0 + 4) * KBYTES < kbytes32;
+      in_k[1] = kbase + (e0 + 5) * KBYTES < kbytes32;
     }
-    const int e0 = even ? ks : ks - 1;
-#pragma unroll
-    for (int t = 0; t < NM; ++t) {
-#pragma unroll
-      for (int r = 0; r < NR; ++r)
-        if (r * RSPAN / NR == t) read_one(rstage, r, xn, wn_);
-#pragma unroll
-      for (int d = 0; d < 2 * LOADS; ++d)
-        if ((d * (2 * NM) / (2 * LOADS) + 1) % (2 * NM) == t + (even ? 0 : NM))
-          fill_one((d & 1) ? pslot1 : pslot0, e0 + 4 + (d & 1), d >> 1);
+    static_for<0, NM>([&](auto T) {
+      constexpr int t = decltype(T)::value;
+      static_for<0, NR>([&](auto R) {
+        constexpr int r = decltype(R)::value;
+        if constexpr (r * RSPAN / NR == t) read_one(std::integral_constant<int, (u + 1) % STAGES>{}, R, xn, wn_);
+      });
+      static_for<0, 2 * LOADS>([&](auto D) {
+        constexpr int d = decltype(D)::value;
+        if constexpr ((d * (2 * NM) / (2 * LOADS) + 1) % (2 * NM) == t + (even ? 0 : NM))
+          fill_one(CHECK, std::integral_constant<int, (e0 + 4 + (d & 1)) % STAGES>{}, std::integral_constant<int, (d >> 1)>{},
+                   std::integral_constant<int, (d & 1)>{}, kbase, std::integral_constant<int, (e0 + 4 + (d & 1)) * KBYTES>{});
+      });
       mfma_slot<ELT, MB, NB>(t, xc, wc, acc);
       __builtin_amdgcn_sched_barrier(0);
-    }
+    });
     FLUXMI_WAITCNT(63, 0);  // the fragments of the next step are in registers (requested long ago)
     __builtin_amdgcn_sched_barrier(0);
   };
 
   // ---- prologue: request k-steps 0..3 as two pairs, wait for the first pair ------------------------
   FLUXMI_WAITCNT(0, 0);  // stores of the previous tile's epilogue
-#pragma unroll
-  for (int s = 0; s < 4; s += 2) {
-    const int s0 = fslot, s1 = next_slot(fslot);
-    fslot = next_slot(s1);
-#pragma unroll
-    for (int q = 0; q < LOADS; ++q) {
-      fill_one(s0, s, q);
-      fill_one(s1, s + 1, q);
-    }
-  }
+  static_for<0, 2>([&](auto P) {
+    constexpr int s = 2 * decltype(P)::value;
+    in_k[0] = s * KBYTES < kbytes32;
+    in_k[1] = (s + 1) * KBYTES < kbytes32;
+    static_for<0, LOADS>([&](auto Q) {
+      fill_one(std::true_type{}, std::integral_constant<int, s>{}, Q, std::integral_constant<int, 0>{}, 0,
+               std::integral_constant<int, s * KBYTES>{});
+      fill_one(std::true_type{}, std::integral_constant<int, s + 1>{}, Q, std::integral_constant<int, 1>{}, 0,
+               std::integral_constant<int, (s + 1) * KBYTES>{});
+    });
+  });
   FLUXMI_WAITCNT(2 * LOADS, 15);
   __builtin_amdgcn_s_barrier();
-  {
-    const uint8_t *stage = smem + rslot * STAGE_BYTES;
-    rslot = next_slot(rslot);
-#pragma unroll
-    for (int r = 0; r < NR; ++r) read_one(stage, r, xa, wa);
-  }
+  static_for<0, NR>([&](auto R) { read_one(std::integral_constant<int, 0>{}, R, xa, wa); });
   FLUXMI_WAITCNT(63, 0);  // in registers before the first step's barrier lets anyone refill that slot
-  // An odd number of k-steps runs one phantom step on zero fragments.
-  for (int ks = 0; ks < nk; ks += 2) {
-    step(ks, true, xa, wa, xb, wb);
-    step(ks + 1, false, xb, wb, xa, wa);
+
+  // ---- main loop: whole trips of ten k-steps; steps past the end of K multiply zeros ----------------
+  // A trip requests k-steps up to 13 past its first one.  While all of those exist the fills need no
+  // checks; the last one or two trips choose between the operand and the zero page per k-step.
+  auto trip_of_ten = [&](auto CHECK, int kbase) {
+    step(CHECK, std::integral_constant<int, 0>{}, kbase, xa, wa, xb, wb);
+    step(CHECK, std::integral_constant<int, 1>{}, kbase, xb, wb, xa, wa);
+    step(CHECK, std::integral_constant<int, 2>{}, kbase, xa, wa, xb, wb);
+    step(CHECK, std::integral_constant<int, 3>{}, kbase, xb, wb, xa, wa);
+    step(CHECK, std::integral_constant<int, 4>{}, kbase, xa, wa, xb, wb);
+    step(CHECK, std::integral_constant<int, 5>{}, kbase, xb, wb, xa, wa);
+    step(CHECK, std::integral_constant<int, 6>{}, kbase, xa, wa, xb, wb);
+    step(CHECK, std::integral_constant<int, 7>{}, kbase, xb, wb, xa, wa);
+    step(CHECK, std::integral_constant<int, 8>{}, kbase, xa, wa, xb, wb);
+    step(CHECK, std::integral_constant<int, 9>{}, kbase, xb, wb, xa, wa);
+  };
+  const int ntrips = (nk + 9) / 10;
+  const int nfast = nk >= 14 ? (nk - 14) / 10 + 1 : 0;  // trips with 10 * trip + 13 < nk
+  int kbase = 0;  // byte offset along K of step 0 of the current trip
+  for (int trip = 0; trip < nfast; ++trip) {
+    trip_of_ten(std::false_type{}, kbase);
+    kbase += 10 * KBYTES;
+  }
+  for (int trip = nfast; trip < ntrips; ++trip) {
+    trip_of_ten(std::true_type{}, kbase);
+    kbase += 10 * KBYTES;
   }
 
   // ---- epilogue ---------------------------------------------------------------------------------
