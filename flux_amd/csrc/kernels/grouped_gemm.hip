@@ -244,15 +244,12 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
   const int64_t xbytes = xrows > 0 ? xrows * c.kbytes : 0xffffffffll;
   const uint8_t *wbase = p.b + (static_cast<int64_t>(e) * p.n + n0) * c.kbytes;
   const int64_t wbytes = static_cast<int64_t>(p.n - n0) * c.kbytes;
-  // The loop runs whole trips of ten k-steps, the surplus ones on zero fragments: a k-step past the end
-  // of K is filled from a page of zeros (every lane at offset 16 * lane).  `in_k[h]` says whether the
-  // h-th k-step of the pair being requested exists.
+  // An odd number of k-steps is rounded up by a phantom step whose fragments come from a page of zeros
+  // (every lane at offset 16 * lane).
   const __amdgpu_buffer_rsrc_t xrsrc = make_rsrc(xbase, xbytes);
   const __amdgpu_buffer_rsrc_t wrsrc = make_rsrc(wbase, wbytes);
   const __amdgpu_buffer_rsrc_t zrsrc = make_rsrc(g_zero_page, 1024);
   const uint32_t zoff = lane * 16;
-  const int kbytes32 = static_cast<int>(c.kbytes);  // K * element size fits 31 bits (K itself is an int32)
-  bool in_k[2] = {true, true};
   uint32_t xoff[XLOADS], woff[WLOADS];
 #pragma unroll
   for (int j = 0; j < XLOADS; ++j) {
@@ -275,19 +272,30 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
   uint8_t *xdst = smem + (XLOADS * wave) * 1024;
   uint8_t *wdst = smem + X_TILE_BYTES + (WLOADS * wave) * 1024;
 
-  // Fill instruction Q of the k-step at byte offset kbase + KOFF of every row (the H-th of its pair), into
-  // ring slot SLOT.  The k offset travels as the scalar offset: an instruction immediate would also be
-  // added to the LDS address.
-  auto fill_one = [&](auto CHECK, auto SLOT, auto Q, auto H, int kbase, auto KOFF) {
-    constexpr int slot = decltype(SLOT)::value, q = decltype(Q)::value, koff = decltype(KOFF)::value;
-    constexpr int h = decltype(H)::value;
-    const bool in = !decltype(CHECK)::value || in_k[h];  // unchecked: the caller knows the k-step exists
+  // Fill instruction Q of the k-step at byte offset kbyte of every row, into ring slot SLOT (compile-time
+  // slot: the LDS address is an immediate).  The k offset travels as the scalar offset: an instruction
+  // immediate would also be added to the LDS address.
+  auto fill_one = [&](auto SLOT, auto Q, int kbyte) {
+    constexpr int slot = decltype(SLOT)::value, q = decltype(Q)::value;
+    if constexpr (q < XLOADS)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(xrsrc, (lds_ptr_t)(xdst + slot * STAGE_BYTES + q * 1024), 16,
+                                               static_cast<int>(xoff[q]), kbyte, 0, 0);
+    else
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(wrsrc, (lds_ptr_t)(wdst + slot * STAGE_BYTES + (q - XLOADS) * 1024), 16,
+                                               static_cast<int>(woff[q - XLOADS]), kbyte, 0, 0);
+  };
+  // Same with a run-time slot, for the last steps of a tile; a k-step past the end of K (the phantom
+  // second half of the last pair of an odd K) is filled from the zero page.
+  auto fill_dyn = [&](int slot, auto Q, int kstep) {
+    constexpr int q = decltype(Q)::value;
+    const bool in = kstep < nk;
+    const int kbyte = in ? kstep * KBYTES : 0;
     if constexpr (q < XLOADS)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(in ? xrsrc : zrsrc, (lds_ptr_t)(xdst + slot * STAGE_BYTES + q * 1024), 16,
-                                               static_cast<int>(in ? xoff[q] : zoff), in ? kbase + koff : 0, 0, 0);
+                                               static_cast<int>(in ? xoff[q] : zoff), kbyte, 0, 0);
     else
       __builtin_amdgcn_raw_ptr_buffer_load_lds(in ? wrsrc : zrsrc, (lds_ptr_t)(wdst + slot * STAGE_BYTES + (q - XLOADS) * 1024),
-                                               16, static_cast<int>(in ? woff[q - XLOADS] : zoff), in ? kbase + koff : 0, 0, 0);
+                                               16, static_cast<int>(in ? woff[q - XLOADS] : zoff), kbyte, 0, 0);
   };
 
   f32x16 acc[MB][NB];
@@ -319,13 +327,20 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
     else xf[q - NB][s] = *reinterpret_cast<const i32x4 *>(xfrag[hi][s] + lo + (q - NB) * 32 * KBYTES);
   };
 
+  auto read_dyn = [&](int slot, auto R, i32x4 (&xf)[MB][2], i32x4 (&wf)[NB][2]) {
+    constexpr int r = decltype(R)::value;
+    constexpr int s = r / LOADS, q = r % LOADS;
+    if constexpr (q < NB) wf[q][s] = *reinterpret_cast<const i32x4 *>(wfrag[0][s] + slot * STAGE_BYTES + q * 32 * KBYTES);
+    else xf[q - NB][s] = *reinterpret_cast<const i32x4 *>(xfrag[0][s] + slot * STAGE_BYTES + (q - NB) * 32 * KBYTES);
+  };
+
   // One k-step, number U within a run of ten (ring of five slots x two fragment sets: after ten steps
   // every slot index and register role repeats, so all of them are compile-time constants here).
   // MFMAs run on `cur` (read during the previous step), the fragments of the next step go into `nxt`,
   // and half of the fills of the pair of steps (E+4, E+5), E = U rounded down to even, are issued:
   // that pair is requested over the two steps E and E+1, row group by row group, both k-steps of a row
   // group back to back (the second one hits the line the first one brought into L1).
-  auto step = [&](auto CHECK, auto U, int kbase, i32x4 (&xc)[MB][2], i32x4 (&wc)[NB][2], i32x4 (&xn)[MB][2], i32x4 (&wn_)[NB][2]) {
+  auto step = [&](auto U, int kbase, i32x4 (&xc)[MB][2], i32x4 (&wc)[NB][2], i32x4 (&xn)[MB][2], i32x4 (&wn_)[NB][2]) {
     constexpr int u = decltype(U)::value;
     constexpr bool even = (u & 1) == 0;
     constexpr int e0 = u & ~1;
@@ -337,10 +352,6 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
     }
     __builtin_amdgcn_s_barrier();     // ... for every wave's share; and everybody is done reading stage u
     __builtin_amdgcn_sched_barrier(0);
-    if constexpr (even && decltype(CHECK)::value) {
-      in_k[0] = kbase + (e0 + 4) * KBYTES < kbytes32;
-      in_k[1] = kbase + (e0 + 5) * KBYTES < kbytes32;
-    }
     static_for<0, NM>([&](auto T) {
       constexpr int t = decltype(T)::value;
       static_for<0, NR>([&](auto R) {
@@ -350,8 +361,8 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
       static_for<0, 2 * LOADS>([&](auto D) {
         constexpr int d = decltype(D)::value;
         if constexpr ((d * (2 * NM) / (2 * LOADS) + 1) % (2 * NM) == t + (even ? 0 : NM))
-          fill_one(CHECK, std::integral_constant<int, (e0 + 4 + (d & 1)) % STAGES>{}, std::integral_constant<int, (d >> 1)>{},
-                   std::integral_constant<int, (d & 1)>{}, kbase, std::integral_constant<int, (e0 + 4 + (d & 1)) * KBYTES>{});
+          fill_one(std::integral_constant<int, (e0 + 4 + (d & 1)) % STAGES>{}, std::integral_constant<int, (d >> 1)>{},
+                   kbase + (e0 + 4 + (d & 1)) * KBYTES);
       });
       mfma_slot<ELT, MB, NB>(t, xc, wc, acc);
       __builtin_amdgcn_sched_barrier(0);
@@ -359,18 +370,47 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
     FLUXMI_WAITCNT(63, 0);  // the fragments of the next step are in registers (requested long ago)
     __builtin_amdgcn_sched_barrier(0);
   };
+  // The same step with run-time ring slots (k-step ks, slot ks % 5), for the last steps of a tile, whose
+  // number is not a multiple of ten.
+  auto step_dyn = [&](int ks, bool even, i32x4 (&xc)[MB][2], i32x4 (&wc)[NB][2], i32x4 (&xn)[MB][2], i32x4 (&wn_)[NB][2]) {
+    if (even) {
+      FLUXMI_WAITCNT(2 * LOADS, 15);
+    } else {
+      FLUXMI_WAITCNT(LOADS, 15);
+    }
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    const int e0 = even ? ks : ks - 1;
+    const int rslot = (ks + 1) % STAGES, pslot0 = (e0 + 4) % STAGES, pslot1 = (e0 + 5) % STAGES;
+    static_for<0, NM>([&](auto T) {
+      constexpr int t = decltype(T)::value;
+      static_for<0, NR>([&](auto R) {
+        constexpr int r = decltype(R)::value;
+        if constexpr (r * RSPAN / NR == t) read_dyn(rslot, R, xn, wn_);
+      });
+      static_for<0, 2 * LOADS>([&](auto D) {
+        constexpr int d = decltype(D)::value;
+        constexpr int at = (d * (2 * NM) / (2 * LOADS) + 1) % (2 * NM);
+        if constexpr (at < NM) {
+          if (at == t && even) fill_dyn((d & 1) ? pslot1 : pslot0, std::integral_constant<int, (d >> 1)>{}, e0 + 4 + (d & 1));
+        } else {
+          if (at - NM == t && !even) fill_dyn((d & 1) ? pslot1 : pslot0, std::integral_constant<int, (d >> 1)>{}, e0 + 4 + (d & 1));
+        }
+      });
+      mfma_slot<ELT, MB, NB>(t, xc, wc, acc);
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    FLUXMI_WAITCNT(63, 0);
+    __builtin_amdgcn_sched_barrier(0);
+  };
 
   // ---- prologue: request k-steps 0..3 as two pairs, wait for the first pair ------------------------
   FLUXMI_WAITCNT(0, 0);  // stores of the previous tile's epilogue
   static_for<0, 2>([&](auto P) {
     constexpr int s = 2 * decltype(P)::value;
-    in_k[0] = s * KBYTES < kbytes32;
-    in_k[1] = (s + 1) * KBYTES < kbytes32;
     static_for<0, LOADS>([&](auto Q) {
-      fill_one(std::true_type{}, std::integral_constant<int, s>{}, Q, std::integral_constant<int, 0>{}, 0,
-               std::integral_constant<int, s * KBYTES>{});
-      fill_one(std::true_type{}, std::integral_constant<int, s + 1>{}, Q, std::integral_constant<int, 1>{}, 0,
-               std::integral_constant<int, (s + 1) * KBYTES>{});
+      fill_dyn(s, Q, s);
+      fill_dyn(s + 1, Q, s + 1);
     });
   });
   FLUXMI_WAITCNT(2 * LOADS, 15);
@@ -378,31 +418,28 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
   static_for<0, NR>([&](auto R) { read_one(std::integral_constant<int, 0>{}, R, xa, wa); });
   FLUXMI_WAITCNT(63, 0);  // in registers before the first step's barrier lets anyone refill that slot
 
-  // ---- main loop: whole trips of ten k-steps; steps past the end of K multiply zeros ----------------
-  // A trip requests k-steps up to 13 past its first one.  While all of those exist the fills need no
-  // checks; the last one or two trips choose between the operand and the zero page per k-step.
-  auto trip_of_ten = [&](auto CHECK, int kbase) {
-    step(CHECK, std::integral_constant<int, 0>{}, kbase, xa, wa, xb, wb);
-    step(CHECK, std::integral_constant<int, 1>{}, kbase, xb, wb, xa, wa);
-    step(CHECK, std::integral_constant<int, 2>{}, kbase, xa, wa, xb, wb);
-    step(CHECK, std::integral_constant<int, 3>{}, kbase, xb, wb, xa, wa);
-    step(CHECK, std::integral_constant<int, 4>{}, kbase, xa, wa, xb, wb);
-    step(CHECK, std::integral_constant<int, 5>{}, kbase, xb, wb, xa, wa);
-    step(CHECK, std::integral_constant<int, 6>{}, kbase, xa, wa, xb, wb);
-    step(CHECK, std::integral_constant<int, 7>{}, kbase, xb, wb, xa, wa);
-    step(CHECK, std::integral_constant<int, 8>{}, kbase, xa, wa, xb, wb);
-    step(CHECK, std::integral_constant<int, 9>{}, kbase, xb, wb, xa, wa);
-  };
-  const int ntrips = (nk + 9) / 10;
+  // ---- main loop ----------------------------------------------------------------------------------
+  // Whole trips of ten k-steps while every k-step a trip requests (up to 13 past its first one) exists,
+  // then the remaining 4 to 23 steps pair by pair with run-time ring slots.  An odd number of k-steps
+  // ends with a phantom step on zero fragments.
   const int nfast = nk >= 14 ? (nk - 14) / 10 + 1 : 0;  // trips with 10 * trip + 13 < nk
   int kbase = 0;  // byte offset along K of step 0 of the current trip
   for (int trip = 0; trip < nfast; ++trip) {
-    trip_of_ten(std::false_type{}, kbase);
+    step(std::integral_constant<int, 0>{}, kbase, xa, wa, xb, wb);
+    step(std::integral_constant<int, 1>{}, kbase, xb, wb, xa, wa);
+    step(std::integral_constant<int, 2>{}, kbase, xa, wa, xb, wb);
+    step(std::integral_constant<int, 3>{}, kbase, xb, wb, xa, wa);
+    step(std::integral_constant<int, 4>{}, kbase, xa, wa, xb, wb);
+    step(std::integral_constant<int, 5>{}, kbase, xb, wb, xa, wa);
+    step(std::integral_constant<int, 6>{}, kbase, xa, wa, xb, wb);
+    step(std::integral_constant<int, 7>{}, kbase, xb, wb, xa, wa);
+    step(std::integral_constant<int, 8>{}, kbase, xa, wa, xb, wb);
+    step(std::integral_constant<int, 9>{}, kbase, xb, wb, xa, wa);
     kbase += 10 * KBYTES;
   }
-  for (int trip = nfast; trip < ntrips; ++trip) {
-    trip_of_ten(std::true_type{}, kbase);
-    kbase += 10 * KBYTES;
+  for (int ks = 10 * nfast; ks < nk; ks += 2) {
+    step_dyn(ks, true, xa, wa, xb, wb);
+    step_dyn(ks + 1, false, xb, wb, xa, wa);
   }
 
   // ---- epilogue ---------------------------------------------------------------------------------
