@@ -135,32 +135,56 @@ struct TileCtx {
   float scalar;
 };
 
+// The kernel's only argument, read again from the kernel argument segment where it is used.  A copy of
+// all of it kept live in scalar registers through the main loop does not fit the register file; the
+// empty asm keeps the compiler from hoisting these loads back to the top of the kernel.
+typedef const __attribute__((address_space(4))) GemmParams *KernArgs;
+__device__ __forceinline__ KernArgs kernel_args() {
+  KernArgs k = (KernArgs)__builtin_amdgcn_kernarg_segment_ptr();
+  asm volatile("" : "+s"(k));
+  return k;
+}
+
 // Epilogue of one wave: acc (32*MB rows x 32*NB columns, MFMA layout) -> scaled, cast, stored.
-// FULL: every row and column of the wave's quarter exists and rows are stored where they are (no
+// Blocks of 64 rows x 32 columns go through one of two 8 KiB LDS windows in fp32 (alternating, so the
+// writes of a block do not wait for the reads of the one before) and come back with eight lanes per
+// row.  FULL: every row and column of the wave's quarter exists and rows are stored where they are (no
 // scatter), so no store is predicated.  OUT_F32 selects the output element type.
 template <int MB, int NB, bool FULL, bool OUT_F32>
-__device__ __forceinline__ void store_tile(const GemmParams &p, uint8_t *window, const TileCtx &c, int e, int row_base,
-                                           int rows_e, int wrow0, int wcol0, const f32x16 (&acc)[MB][NB]) {
-  static_assert(MB % 2 == 0, "the window holds two 32-row blocks");
+__device__ __forceinline__ void store_tile(uint8_t *windows, const TileCtx &c, int e, int row_base, int rows_e,
+                                           int wrow0, int wcol0, const f32x16 (&acc)[MB][NB]) {
+  static_assert(MB % 2 == 0, "a window holds two 32-row blocks");
+  constexpr int ELT_OUT = OUT_F32 ? 4 : 2;
+  const KernArgs p = kernel_args();
   const int lane = c.lane;
   const int h = lane >> 5;
-  const float tile_scale = c.scalar * (p.alpha ? p.alpha[e] : 1.f);
+  const int n = p->n;
+  const float *alpha = p->alpha, *row_scale = p->row_scale, *col_scale = p->col_scale;
+  const float tile_scale = c.scalar * (alpha ? alpha[e] : 1.f);
   float rs[MB];
 #pragma unroll
   for (int i = 0; i < MB; ++i) {
     const int m = wrow0 + i * 32 + (lane & 31);
-    rs[i] = tile_scale * ((p.row_scale && (FULL || m < rows_e)) ? p.row_scale[row_base + m] : 1.f);
+    rs[i] = tile_scale * ((row_scale && (FULL || m < rows_e)) ? row_scale[row_base + m] : 1.f);
   }
   const int rr0 = lane >> 3;  // row of this lane within a group of 8 rows (store phase)
   const int cc = lane & 7;    // its 4-column chunk
+  // Output address of (first row of the wave + rr0, first column of the wave + 4 * cc); blocks and row
+  // groups add multiples of 32 columns and 8 rows.
+  uint8_t *const d = static_cast<uint8_t *>(p->d);
+  uint8_t *dlane = d + (static_cast<int64_t>(row_base + wrow0 + rr0) * n + wcol0 + cc * 4) * ELT_OUT;
+  const int64_t rowgroup_bytes = static_cast<int64_t>(8) * n * ELT_OUT;
+  const int32_t *scatter = FULL ? nullptr : p->scatter_d;
+  const int max_rows = p->max_rows;
+  int block = 0;
 #pragma unroll
   for (int j = 0; j < NB; ++j) {
     const int col = wcol0 + j * 32 + cc * 4;
     float4 cs = make_float4(1.f, 1.f, 1.f, 1.f);
-    if (p.col_scale && (FULL || col < p.n))
-      cs = *reinterpret_cast<const float4 *>(p.col_scale + static_cast<int64_t>(e) * p.n + col);
+    if (col_scale && (FULL || col < n)) cs = *reinterpret_cast<const float4 *>(col_scale + static_cast<int64_t>(e) * n + col);
 #pragma unroll
-    for (int ip = 0; ip < MB / 2; ++ip) {
+    for (int ip = 0; ip < MB / 2; ++ip, ++block) {
+      uint8_t *window = windows + (block & 1) * 8192;
       // write phase: lane holds row (ii*32 + lane%32), columns q*8 + h*4 .. +3 = 16-byte chunk 2q+h
 #pragma unroll
       for (int ii = 0; ii < 2; ++ii) {
@@ -180,25 +204,27 @@ __device__ __forceinline__ void store_tile(const GemmParams &p, uint8_t *window,
         const int rr = it * 8 + rr0;
         v[it] = *reinterpret_cast<const float4 *>(window + rr * 128 + ((cc ^ ((rr >> 1) & 7)) << 4));
       }
+      uint8_t *dp = dlane + (static_cast<int64_t>(ip) * 8) * rowgroup_bytes + j * 32 * ELT_OUT;
 #pragma unroll
-      for (int it = 0; it < 8; ++it) {
-        const int m = wrow0 + ip * 64 + it * 8 + rr0;
-        int64_t drow = row_base + m;
+      for (int it = 0; it < 8; ++it, dp += rowgroup_bytes) {
+        uint8_t *dst = dp;
         if constexpr (!FULL) {
-          if (m >= rows_e || col >= p.n) continue;  // n % 4 == 0: a chunk is all in or all out
-          if (p.scatter_d) {
-            drow = p.scatter_d[row_base + m];
-            if (drow < 0 || drow >= p.max_rows) continue;
+          const int m = wrow0 + ip * 64 + it * 8 + rr0;
+          if (m >= rows_e || col >= n) continue;  // n % 4 == 0: a chunk is all in or all out
+          if (scatter) {
+            const int64_t drow = scatter[row_base + m];
+            if (drow < 0 || drow >= max_rows) continue;
+            dst = d + (drow * n + col) * ELT_OUT;
           }
         }
         const float4 o = make_float4(v[it].x * cs.x, v[it].y * cs.y, v[it].z * cs.z, v[it].w * cs.w);
         if constexpr (OUT_F32) {
-          *reinterpret_cast<float4 *>(static_cast<float *>(p.d) + drow * p.n + col) = o;
+          *reinterpret_cast<float4 *>(dst) = o;
         } else {
           u32x2 b;
           b[0] = pack_bf16x2(o.x, o.y);
           b[1] = pack_bf16x2(o.z, o.w);
-          *reinterpret_cast<u32x2 *>(static_cast<uint16_t *>(p.d) + drow * p.n + col) = b;
+          *reinterpret_cast<u32x2 *>(dst) = b;
         }
       }
     }
@@ -445,16 +471,20 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
   // ---- epilogue ---------------------------------------------------------------------------------
   FLUXMI_WAITCNT(0, 0);          // this wave's trailing ring fills have landed
   __builtin_amdgcn_s_barrier();  // ... and everybody else's; nobody reads the ring any more
-  uint8_t *window = smem + wave * 8192;
+  uint8_t *windows = smem + wave * 16384;  // two 8 KiB windows per wave
   const int wrow0 = m0 + wm * (32 * MB);
   const int wcol0 = n0 + wn * (32 * NB);
-  const bool full = wrow0 + 32 * MB <= rows_e && wcol0 + 32 * NB <= p.n && p.scatter_d == nullptr;
-  if (full) {
-    if (p.d_fp32) store_tile<MB, NB, true, true>(p, window, c, e, row_base, rows_e, wrow0, wcol0, acc);
-    else store_tile<MB, NB, true, false>(p, window, c, e, row_base, rows_e, wrow0, wcol0, acc);
-  } else {
-    if (p.d_fp32) store_tile<MB, NB, false, true>(p, window, c, e, row_base, rows_e, wrow0, wcol0, acc);
-    else store_tile<MB, NB, false, false>(p, window, c, e, row_base, rows_e, wrow0, wcol0, acc);
+  {
+    const KernArgs pe = kernel_args();
+    const bool full = wrow0 + 32 * MB <= rows_e && wcol0 + 32 * NB <= pe->n && pe->scatter_d == nullptr;
+    const bool out_f32 = pe->d_fp32 != 0;
+    if (full) {
+      if (out_f32) store_tile<MB, NB, true, true>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
+      else store_tile<MB, NB, true, false>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
+    } else {
+      if (out_f32) store_tile<MB, NB, false, true>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
+      else store_tile<MB, NB, false, false>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
+    }
   }
   __builtin_amdgcn_s_barrier();  // the LDS windows are free again before the next tile's fills start
 }
