@@ -145,6 +145,15 @@ __device__ __forceinline__ KernArgs kernel_args() {
   return k;
 }
 
+// One accumulator element, moved out of its accumulation register at the point of use.  Left to itself
+// the compiler copies all 256 of them into vector registers ahead of the epilogue's branches, which
+// does not fit.
+__device__ __forceinline__ float acc_read(float a) {
+  float v;
+  asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(a));
+  return v;
+}
+
 // Epilogue of one wave: acc (32*MB rows x 32*NB columns, MFMA layout) -> scaled, cast, stored.
 // Blocks of 64 rows x 32 columns go through one of two 8 KiB LDS windows in fp32 (alternating, so the
 // writes of a block do not wait for the reads of the one before) and come back with eight lanes per
@@ -192,8 +201,8 @@ __device__ __forceinline__ void store_tile(uint8_t *windows, const TileCtx &c, i
         const int r = ii * 32 + (lane & 31);
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const float4 v = make_float4(acc[i][j][4 * q + 0] * rs[i], acc[i][j][4 * q + 1] * rs[i],
-                                       acc[i][j][4 * q + 2] * rs[i], acc[i][j][4 * q + 3] * rs[i]);
+          const float4 v = make_float4(acc_read(acc[i][j][4 * q + 0]) * rs[i], acc_read(acc[i][j][4 * q + 1]) * rs[i],
+                                       acc_read(acc[i][j][4 * q + 2]) * rs[i], acc_read(acc[i][j][4 * q + 3]) * rs[i]);
           *reinterpret_cast<float4 *>(window + r * 128 + (((2 * q + h) ^ ((r >> 1) & 7)) << 4)) = v;
         }
       }
