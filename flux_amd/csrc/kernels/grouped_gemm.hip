@@ -256,8 +256,9 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const uint8_t *base,
 }
 
 // One output tile of (64*MB) rows x (64*NB) columns at rows [m0, ..) of expert e, columns [n0, ..).
-// (MB, NB) = (4, 4) is the macro tile; (4, 2) and (2, 2) are the 256x128 and 128x128 pieces a tile of
-// the last, partly filled round is cut into.  Waves are laid out 2 x 2.
+// (MB, NB) = (4, 4) is the macro tile, (2, 4) its upper half (for the last rows of an expert); (4, 2) and
+// (2, 2) are the 256x128 and 128x128 pieces a tile of the last, partly filled round is cut into.  Waves
+// are laid out 2 x 2.
 template <int ELT, int MB, int NB>
 __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, const TileCtx &c, int e, int row_base,
                                           int rows_e, int m0, int n0) {
@@ -606,7 +607,9 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
     int n0 = nt * BN;
 
     if (item < full_items || pieces == 1) {
-      gemm_tile<ELT, 4, 4>(p, smem, c, e, row_base, rows_e, m0, n0);
+      // The last row tile of an expert is run 128 rows high when that covers its rows.
+      if (rows_e - m0 > 128) gemm_tile<ELT, 4, 4>(p, smem, c, e, row_base, rows_e, m0, n0);
+      else gemm_tile<ELT, 2, 4>(p, smem, c, e, row_base, rows_e, m0, n0);
     } else if (pieces == 2) {
       n0 += piece * 128;
       if (n0 < p.n) gemm_tile<ELT, 4, 2>(p, smem, c, e, row_base, rows_e, m0, n0);
