@@ -158,8 +158,9 @@ __device__ __forceinline__ float acc_read(float a) {
 // Blocks of 64 rows x 32 columns go through one of two 8 KiB LDS windows in fp32 (alternating, so the
 // writes of a block do not wait for the reads of the one before) and come back with eight lanes per
 // row.  FULL: every row and column of the wave's quarter exists and rows are stored where they are (no
-// scatter), so no store is predicated.  OUT_F32 selects the output element type.
-template <int MB, int NB, bool FULL, bool OUT_F32>
+// scatter), so no store is predicated.  OUT_F32 selects the output element type.  !SCALED: every scale
+// factor is 1 and the multiplications are left out.
+template <int MB, int NB, bool FULL, bool OUT_F32, bool SCALED>
 __device__ __forceinline__ void store_tile(uint8_t *windows, const TileCtx &c, int e, int row_base, int rows_e,
                                            int wrow0, int wcol0, const f32x16 (&acc)[MB][NB]) {
   static_assert(MB % 2 == 0, "a window holds two 32-row blocks");
@@ -201,8 +202,9 @@ __device__ __forceinline__ void store_tile(uint8_t *windows, const TileCtx &c, i
         const int r = ii * 32 + (lane & 31);
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const float4 v = make_float4(acc_read(acc[i][j][4 * q + 0]) * rs[i], acc_read(acc[i][j][4 * q + 1]) * rs[i],
-                                       acc_read(acc[i][j][4 * q + 2]) * rs[i], acc_read(acc[i][j][4 * q + 3]) * rs[i]);
+          float4 v = make_float4(acc_read(acc[i][j][4 * q + 0]), acc_read(acc[i][j][4 * q + 1]),
+                                 acc_read(acc[i][j][4 * q + 2]), acc_read(acc[i][j][4 * q + 3]));
+          if constexpr (SCALED) v = make_float4(v.x * rs[i], v.y * rs[i], v.z * rs[i], v.w * rs[i]);
           *reinterpret_cast<float4 *>(window + r * 128 + (((2 * q + h) ^ ((r >> 1) & 7)) << 4)) = v;
         }
       }
@@ -226,7 +228,8 @@ __device__ __forceinline__ void store_tile(uint8_t *windows, const TileCtx &c, i
             dst = d + (drow * n + col) * ELT_OUT;
           }
         }
-        const float4 o = make_float4(v[it].x * cs.x, v[it].y * cs.y, v[it].z * cs.z, v[it].w * cs.w);
+        float4 o = v[it];
+        if constexpr (SCALED) o = make_float4(o.x * cs.x, o.y * cs.y, o.z * cs.z, o.w * cs.w);
         if constexpr (OUT_F32) {
           *reinterpret_cast<float4 *>(dst) = o;
         } else {
@@ -488,12 +491,16 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
     const KernArgs pe = kernel_args();
     const bool full = wrow0 + 32 * MB <= rows_e && wcol0 + 32 * NB <= pe->n && pe->scatter_d == nullptr;
     const bool out_f32 = pe->d_fp32 != 0;
-    if (full) {
-      if (out_f32) store_tile<MB, NB, true, true>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
-      else store_tile<MB, NB, true, false>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
+    const bool scaled = !(c.scalar == 1.f && pe->alpha == nullptr && pe->row_scale == nullptr && pe->col_scale == nullptr);
+    if (full && !scaled) {
+      if (out_f32) store_tile<MB, NB, true, true, false>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
+      else store_tile<MB, NB, true, false, false>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
+    } else if (full) {
+      if (out_f32) store_tile<MB, NB, true, true, true>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
+      else store_tile<MB, NB, true, false, true>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
     } else {
-      if (out_f32) store_tile<MB, NB, false, true>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
-      else store_tile<MB, NB, false, false>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
+      if (out_f32) store_tile<MB, NB, false, true, true>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
+      else store_tile<MB, NB, false, false, true>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
     }
   }
   __builtin_amdgcn_s_barrier();  // the LDS windows are free again before the next tile's fills start
