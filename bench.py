@@ -195,6 +195,24 @@ def main():
         kernels["gemm_fp8_c5_layer1"] = {"ms": round(t_f8, 4), "tflops": round(f_f8 / t_f8 * 1e-9, 1),
                                          "frac_fp8_peak": round(f_f8 / t_f8 * 1e-9 / PEAK_FP8_TFLOPS, 4)}
         del a8, b8, d5
+        # The same two C3 GEMMs as a loop of library GEMMs (torch.mm = hipBLASLt), one per expert, on rows that
+        # are already gathered and contiguous: the path a port without a grouped kernel would take.  Reported
+        # beside the grouped kernel for comparison; not part of the step.
+        xg = torch.randn(m, h, generator=gen, device=dev).to(torch.bfloat16)
+        bounds = [0] + [int(v) for v in wl.splits.cumsum()]
+
+        def lib_loop(src, wts, dst):
+            for ei in range(e):
+                r0, r1 = bounds[ei], bounds[ei + 1]
+                if r1 > r0:
+                    torch.mm(src[r0:r1], wts[ei].t(), out=dst[r0:r1])
+
+        zl = torch.empty(m, h, dtype=torch.bfloat16, device=dev)
+        for name, fn in (("library_gemm_loop_layer0", lambda: lib_loop(xg, w1, y)),
+                         ("library_gemm_loop_layer1", lambda: lib_loop(y, w2, zl))):
+            t_l = time_loop(torch, fn, 20)
+            kernels[name] = {"ms": round(t_l, 4), "tflops": round(gemm_flops / t_l * 1e-9, 1)}
+        del xg, zl
 
     if a.calib_copy:
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()

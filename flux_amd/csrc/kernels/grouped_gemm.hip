@@ -694,12 +694,17 @@ __global__ __launch_bounds__(256) void grouped_gemm_generic_kernel(const GemmPar
   }
 }
 
+// Shapes the MFMA kernel takes: K a multiple of 64 bytes, N a multiple of 4, aligned pointers, and
+// operands its 32-bit buffer offsets can span (a gathered A as a whole, 256 rows of an ungathered A, one
+// expert's weights).  Everything else runs the generic kernel.
 bool mfma_path_ok(const fluxmi_grouped_gemm_args *a) {
   const int elt = a->dtype == FLUXMI_BF16 ? 2 : 1;
   const int64_t kbytes = static_cast<int64_t>(a->k) * elt;
+  const int64_t span = 0xffffffffll;
+  const bool a_fits = a->gather_a ? (a->a_rows > 0 && a->a_rows * kbytes <= span) : BM * kbytes <= span;
   return kbytes % KBYTES == 0 && kbytes >= KBYTES && a->n % 4 == 0 && aligned16(a->a) &&
          aligned16(a->b) && (reinterpret_cast<uintptr_t>(a->d) & (a->d_fp32 ? 15u : 7u)) == 0 &&
-         (a->col_scale == nullptr || aligned16(a->col_scale));
+         (a->col_scale == nullptr || aligned16(a->col_scale)) && a_fits && a->n * kbytes <= span;
 }
 
 template <int ELT>

@@ -93,7 +93,7 @@ typedef struct fluxmi_grouped_gemm_args {
   int32_t max_rows;      /* upper bound on the number of sorted rows */
   int32_t n;             /* N, columns of D / rows of each B[e] */
   int32_t k;             /* K */
-  int32_t a_rows;        /* rows of A when gather_a is given: entries are clamped into [0, a_rows); 0 = trust them */
+  int32_t a_rows;        /* rows of A when gather_a is given: entries are clamped into [0, a_rows); 0 = trust them (and take the slow generic kernel: the MFMA kernel needs the extent of a gathered A) */
   const void *a;         /* [rows_a, K] */
   const void *b;         /* [E, N, K] */
   void *d;               /* [max_rows, N] bf16 (fp32 when d_fp32 != 0) */
