@@ -93,17 +93,33 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 // Source of the ring fills of a k-step past the end of K: every lane reads 16 zero bytes.
 __device__ __attribute__((aligned(1024))) const uint8_t g_zero_page[1024] = {};
 
-// MFMA number t of a k-step.  bf16: 2 * MB * NB instructions of 32x32x16, the two 16-element halves of
-// the step one after the other.  fp8: MB * NB instructions of 32x32x64 (both 16-byte chunks at once).
-template <int ELT, int MB, int NB>
-__device__ __forceinline__ void mfma_slot(int t, const i32x4 (&xf)[MB][2], const i32x4 (&wf)[NB][2],
-                                          f32x16 (&acc)[MB][NB]) {
+// MFMA geometry per element type.  bf16 uses v_mfma_f32_16x16x32_bf16: one instruction consumes a whole
+// k-step (32 elements) of a 16-row block of each operand, i.e. one 16-byte fragment register set per
+// block, and accumulates a 16x16 block in 4 registers.  At the same FLOP rate as the 32x32x16 form it
+// moves half the accumulator bytes per FLOP through the register file, and measured under the board's
+// power limit that is worth 18 % of sustained MFMA throughput.  fp8 uses the 32x32x64 f8f6f4 form: two
+// 16-byte fragment chunks per 32-row block and k-step, 16 accumulator registers per block.
+template <int ELT>
+struct Geom {
+  static constexpr int BLK = ELT == 2 ? 16 : 32;  // rows (columns) of an operand block
+  static constexpr int NCH = ELT == 2 ? 1 : 2;    // 16-byte fragment chunks per block and k-step
+  static constexpr int NACC = BLK * BLK / 64;     // accumulator registers per block
+  typedef float Acc __attribute__((ext_vector_type(NACC)));
+};
+
+// MFMA number t of a k-step over MBK x NBK blocks: block row i = t / NBK, block column j = t % NBK.
+template <int ELT, int MBK, int NBK>
+__device__ __forceinline__ void mfma_slot(int t, const i32x4 (&xf)[MBK][Geom<ELT>::NCH], const i32x4 (&wf)[NBK][Geom<ELT>::NCH],
+                                          typename Geom<ELT>::Acc (&acc)[MBK][NBK]) {
+  const int i = t / NBK, j = t % NBK;
   if constexpr (ELT == 2) {
-    const int s = t / (MB * NB), i = (t % (MB * NB)) / NB, j = t % NB;
-    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, wf[j][s]),
-                                                        __builtin_bit_cast(bf16x8, xf[i][s]), acc[i][j], 0, 0, 0);
+    // Written as asm to pin the accumulators to the accumulation registers: given the builtin, the
+    // register allocator spreads the 64 four-register accumulators over both register files and shuffles
+    // them at the loop's back edge.  Every accumulator is touched once per k-step, 63 MFMAs apart, and
+    // the fragment operands come from LDS reads the compiler still tracks, so no hazard needs software
+    // wait states here.
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(wf[j][0]), "v"(xf[i][0]));
   } else {
-    const int i = t / NB, j = t % NB;
     i32x8 wa, xa;
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
@@ -157,13 +173,16 @@ __device__ __forceinline__ float acc_read(float a) {
 // Epilogue of one wave: acc (32*MB rows x 32*NB columns, MFMA layout) -> scaled, cast, stored.
 // Blocks of 64 rows x 32 columns go through one of two 8 KiB LDS windows in fp32 (alternating, so the
 // writes of a block do not wait for the reads of the one before) and come back with eight lanes per
-// row.  FULL: every row and column of the wave's quarter exists and rows are stored where they are (no
+// row (j below counts 32-column groups, ip 64-row groups).  FULL: every row and column of the wave's quarter exists and rows are stored where they are (no
 // scatter), so no store is predicated.  OUT_F32 selects the output element type.  !SCALED: every scale
 // factor is 1 and the multiplications are left out.
-template <int MB, int NB, bool FULL, bool OUT_F32, bool SCALED>
-__device__ __forceinline__ void store_tile(uint8_t *windows, const TileCtx &c, int e, int row_base, int rows_e,
-                                           int wrow0, int wcol0, const f32x16 (&acc)[MB][NB]) {
-  static_assert(MB % 2 == 0, "a window holds two 32-row blocks");
+template <int ELT, int MB, int NB, bool FULL, bool OUT_F32, bool SCALED>
+__device__ __forceinline__ void store_tile(uint8_t *windows, const TileCtx &c, int e, int row_base, int rows_e, int wrow0,
+                                           int wcol0,
+                                           const typename Geom<ELT>::Acc (&acc)[32 * MB / Geom<ELT>::BLK][32 * NB / Geom<ELT>::BLK]) {
+  static_assert(MB % 2 == 0, "a window holds 64 rows");
+  constexpr int BLK = Geom<ELT>::BLK;
+  constexpr int MBK = 32 * MB / BLK;
   constexpr int ELT_OUT = OUT_F32 ? 4 : 2;
   const KernArgs p = kernel_args();
   const int lane = c.lane;
@@ -171,10 +190,10 @@ __device__ __forceinline__ void store_tile(uint8_t *windows, const TileCtx &c, i
   const int n = p->n;
   const float *alpha = p->alpha, *row_scale = p->row_scale, *col_scale = p->col_scale;
   const float tile_scale = c.scalar * (alpha ? alpha[e] : 1.f);
-  float rs[MB];
+  float rs[MBK];  // scale of this lane's row in each block row
 #pragma unroll
-  for (int i = 0; i < MB; ++i) {
-    const int m = wrow0 + i * 32 + (lane & 31);
+  for (int i = 0; i < MBK; ++i) {
+    const int m = wrow0 + i * BLK + (lane & (BLK - 1));
     rs[i] = tile_scale * ((row_scale && (FULL || m < rows_e)) ? row_scale[row_base + m] : 1.f);
   }
   const int rr0 = lane >> 3;  // row of this lane within a group of 8 rows (store phase)
@@ -195,17 +214,23 @@ __device__ __forceinline__ void store_tile(uint8_t *windows, const TileCtx &c, i
 #pragma unroll
     for (int ip = 0; ip < MB / 2; ++ip, ++block) {
       uint8_t *window = windows + (block & 1) * 8192;
-      // write phase: lane holds row (ii*32 + lane%32), columns q*8 + h*4 .. +3 = 16-byte chunk 2q+h
+      // write phase.  A lane holds one row of a block and groups of 4 consecutive columns of it: with
+      // 16x16 blocks one group, columns 4 * (lane / 16); with 32x32 blocks four, columns 8q + 4 * (lane / 32).
 #pragma unroll
-      for (int ii = 0; ii < 2; ++ii) {
-        const int i = ip * 2 + ii;
-        const int r = ii * 32 + (lane & 31);
+      for (int ii = 0; ii < 64 / BLK; ++ii) {
+        const int i = ip * (64 / BLK) + ii;
+        const int r = ii * BLK + (lane & (BLK - 1));
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          float4 v = make_float4(acc_read(acc[i][j][4 * q + 0]), acc_read(acc[i][j][4 * q + 1]),
-                                 acc_read(acc[i][j][4 * q + 2]), acc_read(acc[i][j][4 * q + 3]));
-          if constexpr (SCALED) v = make_float4(v.x * rs[i], v.y * rs[i], v.z * rs[i], v.w * rs[i]);
-          *reinterpret_cast<float4 *>(window + r * 128 + (((2 * q + h) ^ ((r >> 1) & 7)) << 4)) = v;
+        for (int jj = 0; jj < 32 / BLK; ++jj) {
+          const int jb = j * (32 / BLK) + jj;
+#pragma unroll
+          for (int q = 0; q < Geom<ELT>::NACC / 4; ++q) {
+            const int chunk = BLK == 32 ? 2 * q + h : jj * 4 + (lane >> 4);
+            float4 v = make_float4(acc_read(acc[i][jb][4 * q + 0]), acc_read(acc[i][jb][4 * q + 1]),
+                                   acc_read(acc[i][jb][4 * q + 2]), acc_read(acc[i][jb][4 * q + 3]));
+            if constexpr (SCALED) v = make_float4(v.x * rs[i], v.y * rs[i], v.z * rs[i], v.w * rs[i]);
+            *reinterpret_cast<float4 *>(window + r * 128 + ((chunk ^ ((r >> 1) & 7)) << 4)) = v;
+          }
         }
       }
       // store phase: 8 lanes per row, 8 rows per instruction
@@ -268,8 +293,10 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
   constexpr int XLOADS = MB;           // direct-to-LDS instructions per wave per stage, X tile
   constexpr int WLOADS = NB;           // same, W tile
   constexpr int LOADS = XLOADS + WLOADS;
-  constexpr int NR = LOADS * 2;        // fragment reads per k-step
-  constexpr int NM = MB * NB * (ELT == 2 ? 2 : 1);  // MFMAs per k-step
+  constexpr int BLK = Geom<ELT>::BLK, NCH = Geom<ELT>::NCH;
+  constexpr int MBK = 32 * MB / BLK, NBK = 32 * NB / BLK;  // operand blocks of a wave
+  constexpr int NR = (MBK + NBK) * NCH;  // fragment reads per k-step (16 bytes per lane each)
+  constexpr int NM = MBK * NBK;          // MFMAs per k-step
   constexpr int RSPAN = NM / 2;        // MFMA slots over which the fragment reads of a step are spread
   const int wave = c.wave, lane = c.lane, wm = c.wm, wn = c.wn, nk = c.nk;
 
@@ -337,40 +364,40 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
                                                16, static_cast<int>(in ? woff[q - XLOADS] : zoff), kbyte, 0, 0);
   };
 
-  f32x16 acc[MB][NB];
+  typename Geom<ELT>::Acc acc[MBK][NBK];
 #pragma unroll
-  for (int i = 0; i < MB; ++i)
+  for (int i = 0; i < MBK; ++i)
 #pragma unroll
-    for (int j = 0; j < NB; ++j)
+    for (int j = 0; j < NBK; ++j)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+      for (int v = 0; v < Geom<ELT>::NACC; ++v) acc[i][j][v] = 0.f;
 
   // Fragment addresses: per lane and 16-byte chunk s a base for each operand; a stage and block add a
   // compile-time offset.  LDS instructions carry 16 bits of offset, so three bases 64 KiB apart.
-  const uint8_t *xfrag[3][2], *wfrag[3][2];
+  const uint8_t *xfrag[3][NCH], *wfrag[3][NCH];
 #pragma unroll
   for (int hi = 0; hi < 3; ++hi)
 #pragma unroll
-    for (int s = 0; s < 2; ++s) {
+    for (int s = 0; s < NCH; ++s) {
       xfrag[hi][s] = smem + hi * 65536 + wm * (32 * MB) * KBYTES + c.frag_off[s];
       wfrag[hi][s] = smem + hi * 65536 + X_TILE_BYTES + wn * (32 * NB) * KBYTES + c.frag_off[s];
     }
-  i32x4 xa[MB][2], wa[NB][2], xb[MB][2], wb[NB][2];
-  // Fragment read R of the k-step in ring slot SLOT: chunk s = R / LOADS of W block q (q < NB) or of
-  // X block q - NB.
-  auto read_one = [&](auto SLOT, auto R, i32x4 (&xf)[MB][2], i32x4 (&wf)[NB][2]) {
+  i32x4 xa[MBK][NCH], wa[NBK][NCH], xb[MBK][NCH], wb[NBK][NCH];
+  // Fragment read R of the k-step in ring slot SLOT: chunk s = R / (MBK + NBK) of W block q (q < NBK) or of
+  // X block q - NBK.
+  auto read_one = [&](auto SLOT, auto R, i32x4 (&xf)[MBK][NCH], i32x4 (&wf)[NBK][NCH]) {
     constexpr int slot = decltype(SLOT)::value, r = decltype(R)::value;
-    constexpr int s = r / LOADS, q = r % LOADS;
+    constexpr int s = r / (MBK + NBK), q = r % (MBK + NBK);
     constexpr int hi = (slot * STAGE_BYTES) / 65536, lo = (slot * STAGE_BYTES) % 65536;
-    if constexpr (q < NB) wf[q][s] = *reinterpret_cast<const i32x4 *>(wfrag[hi][s] + lo + q * 32 * KBYTES);
-    else xf[q - NB][s] = *reinterpret_cast<const i32x4 *>(xfrag[hi][s] + lo + (q - NB) * 32 * KBYTES);
+    if constexpr (q < NBK) wf[q][s] = *reinterpret_cast<const i32x4 *>(wfrag[hi][s] + lo + q * BLK * KBYTES);
+    else xf[q - NBK][s] = *reinterpret_cast<const i32x4 *>(xfrag[hi][s] + lo + (q - NBK) * BLK * KBYTES);
   };
 
-  auto read_dyn = [&](int slot, auto R, i32x4 (&xf)[MB][2], i32x4 (&wf)[NB][2]) {
+  auto read_dyn = [&](int slot, auto R, i32x4 (&xf)[MBK][NCH], i32x4 (&wf)[NBK][NCH]) {
     constexpr int r = decltype(R)::value;
-    constexpr int s = r / LOADS, q = r % LOADS;
-    if constexpr (q < NB) wf[q][s] = *reinterpret_cast<const i32x4 *>(wfrag[0][s] + slot * STAGE_BYTES + q * 32 * KBYTES);
-    else xf[q - NB][s] = *reinterpret_cast<const i32x4 *>(xfrag[0][s] + slot * STAGE_BYTES + (q - NB) * 32 * KBYTES);
+    constexpr int s = r / (MBK + NBK), q = r % (MBK + NBK);
+    if constexpr (q < NBK) wf[q][s] = *reinterpret_cast<const i32x4 *>(wfrag[0][s] + slot * STAGE_BYTES + q * BLK * KBYTES);
+    else xf[q - NBK][s] = *reinterpret_cast<const i32x4 *>(xfrag[0][s] + slot * STAGE_BYTES + (q - NBK) * BLK * KBYTES);
   };
 
   // One k-step, number U within a run of ten (ring of five slots x two fragment sets: after ten steps
@@ -379,7 +406,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
   // and half of the fills of the pair of steps (E+4, E+5), E = U rounded down to even, are issued:
   // that pair is requested over the two steps E and E+1, row group by row group, both k-steps of a row
   // group back to back (the second one hits the line the first one brought into L1).
-  auto step = [&](auto U, int kbase, i32x4 (&xc)[MB][2], i32x4 (&wc)[NB][2], i32x4 (&xn)[MB][2], i32x4 (&wn_)[NB][2]) {
+  auto step = [&](auto U, int kbase, i32x4 (&xc)[MBK][NCH], i32x4 (&wc)[NBK][NCH], i32x4 (&xn)[MBK][NCH], i32x4 (&wn_)[NBK][NCH]) {
     constexpr int u = decltype(U)::value;
     constexpr bool even = (u & 1) == 0;
     constexpr int e0 = u & ~1;
@@ -403,7 +430,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
           fill_one(std::integral_constant<int, (e0 + 4 + (d & 1)) % STAGES>{}, std::integral_constant<int, (d >> 1)>{},
                    kbase + (e0 + 4 + (d & 1)) * KBYTES);
       });
-      mfma_slot<ELT, MB, NB>(t, xc, wc, acc);
+      mfma_slot<ELT, MBK, NBK>(t, xc, wc, acc);
       __builtin_amdgcn_sched_barrier(0);
     });
     FLUXMI_WAITCNT(63, 0);  // the fragments of the next step are in registers (requested long ago)
@@ -411,7 +438,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
   };
   // The same step with run-time ring slots (k-step ks, slot ks % 5), for the last steps of a tile, whose
   // number is not a multiple of ten.
-  auto step_dyn = [&](int ks, bool even, i32x4 (&xc)[MB][2], i32x4 (&wc)[NB][2], i32x4 (&xn)[MB][2], i32x4 (&wn_)[NB][2]) {
+  auto step_dyn = [&](int ks, bool even, i32x4 (&xc)[MBK][NCH], i32x4 (&wc)[NBK][NCH], i32x4 (&xn)[MBK][NCH], i32x4 (&wn_)[NBK][NCH]) {
     if (even) {
       FLUXMI_WAITCNT(2 * LOADS, 15);
     } else {
@@ -436,7 +463,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
           if (at - NM == t && !even) fill_dyn((d & 1) ? pslot1 : pslot0, std::integral_constant<int, (d >> 1)>{}, e0 + 4 + (d & 1));
         }
       });
-      mfma_slot<ELT, MB, NB>(t, xc, wc, acc);
+      mfma_slot<ELT, MBK, NBK>(t, xc, wc, acc);
       __builtin_amdgcn_sched_barrier(0);
     });
     FLUXMI_WAITCNT(63, 0);
@@ -493,14 +520,14 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
     const bool out_f32 = pe->d_fp32 != 0;
     const bool scaled = !(c.scalar == 1.f && pe->alpha == nullptr && pe->row_scale == nullptr && pe->col_scale == nullptr);
     if (full && !scaled) {
-      if (out_f32) store_tile<MB, NB, true, true, false>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
-      else store_tile<MB, NB, true, false, false>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
+      if (out_f32) store_tile<ELT, MB, NB, true, true, false>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
+      else store_tile<ELT, MB, NB, true, false, false>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
     } else if (full) {
-      if (out_f32) store_tile<MB, NB, true, true, true>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
-      else store_tile<MB, NB, true, false, true>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
+      if (out_f32) store_tile<ELT, MB, NB, true, true, true>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
+      else store_tile<ELT, MB, NB, true, false, true>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
     } else {
-      if (out_f32) store_tile<MB, NB, false, true, true>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
-      else store_tile<MB, NB, false, false, true>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
+      if (out_f32) store_tile<ELT, MB, NB, false, true, true>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
+      else store_tile<ELT, MB, NB, false, false, true>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
     }
   }
   __builtin_amdgcn_s_barrier();  // the LDS windows are free again before the next tile's fills start
@@ -529,12 +556,20 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
   // superline 4q + (l >> 4), slot l & 15, i.e. row 16q + (l >> 2), chunk (l & 3) ^ ((l >> 4) & 3).
   c.fill_row = lane >> 2;
   c.fill_chunk = (lane & 3) ^ ((lane >> 4) & 3);
-  // Fragment reads: lane l reads row (l & 31) of a 32-row block, chunk c(s) for s = 0,1.
+  // Fragment reads.  bf16: lane l reads row (l & 15) of a 16-row block, chunk l >> 4 (the four chunks of
+  // a row are the 32 k-elements of one MFMA).  fp8: row (l & 31) of a 32-row block, chunks 2 * (l >> 5) + s.
+  if (ELT == 2) {
+    const int r = lane & 15, ch = lane >> 4;
+    const int slot = ((r & 3) << 2) | (ch ^ ((r >> 2) & 3));
+    c.frag_off[0] = (r >> 2) * 256 + slot * 16;
+    c.frag_off[1] = 0;
+  } else {
 #pragma unroll
-  for (int s = 0; s < 2; ++s) {
-    const int ch = ELT == 2 ? 2 * s + (lane >> 5) : 2 * (lane >> 5) + s;
-    const int slot = ((lane & 3) << 2) | (ch ^ ((lane >> 2) & 3));
-    c.frag_off[s] = ((lane & 31) >> 2) * 256 + slot * 16;
+    for (int s = 0; s < 2; ++s) {
+      const int ch = 2 * (lane >> 5) + s;
+      const int slot = ((lane & 3) << 2) | (ch ^ ((lane >> 2) & 3));
+      c.frag_off[s] = ((lane & 31) >> 2) * 256 + slot * 16;
+    }
   }
   c.scalar = p.scalar;
   if (p.scalar_dev) c.scalar *= p.scalar_dev[0];
