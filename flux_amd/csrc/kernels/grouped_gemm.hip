@@ -1,667 +1,9 @@
-// Grouped GEMM over ragged per-expert row counts: D[r,:] = scale(r,:) * A[gather(r),:] @ B[e(r)]^T.
-//
-// Persistent kernel, one 256-thread workgroup (4 waves, one per SIMD) per CU, macro tile 256 rows x 256
-// columns, k-step of 64 bytes per row (32 bf16 or 64 fp8).  Both operand tiles are staged in LDS by
-// direct-to-LDS global loads (no register staging) in a ring of five 32 KiB stages; the row gather of A
-// is folded into the per-lane global address of those loads.  Each wave owns a 128 x 128 quarter of the
-// macro tile (4x4 MFMA blocks of 32x32, 256 fp32 accumulator registers) and runs a software pipeline
-// of its own: while the MFMAs of k-step s run on one set of fragment registers, the fragments of step
-// s+1 are read from LDS into a second set and the ring fills of steps s+4 / s+5 are issued, all in a
-// fixed interleaving (one fragment read per MFMA over the first half of the step, one fill every
-// fourth MFMA).  One workgroup barrier per k-step publishes the landed stage.
-//
-// Ring fills are issued in pairs of k-steps: the two 64-byte halves of a 128-byte line are requested
-// back to back (they go to different stages), so the second request hits the line the first one
-// brought into the vector L1 and L2 sees one request per line instead of two.
-//
-// The MFMA "A" operand is the weight fragment and the "B" operand the activation fragment, i.e. the
-// hardware computes D^T blocks: a lane then holds, for one output row, four consecutive output columns
-// per accumulator quad.  The epilogue passes each 64-row x 32-column block through a wave-private LDS
-// window in fp32 and reads it back with eight lanes per row, so that one store instruction writes 64
-// (bf16) or 128 (fp32) contiguous bytes of each row.
-//
-// Tile schedule: every wave walks the device-resident `splits` with scalar loads, in step with the
-// increasing logical tile ids of its workgroup; ids are assigned so that the workgroups of one XCD
-// (those with equal blockIdx % 8) take a run of consecutive tiles; tiles of an expert are ordered in
-// groups of at most 8 row tiles, each group walked column-major over the weight panels, so an XCD's L2
-// sees a few weight panels shared by the row tiles of a group.
-#include <cstdlib>
-#include <type_traits>
-
-#include "common.hpp"
+// Grouped GEMM entry point: argument checks, choice between the MFMA kernel and the generic kernel, and
+// the generic kernel itself.  The MFMA kernel lives in grouped_gemm_kernel.hpp.
+#include "grouped_gemm.hpp"
 
 namespace fluxmi {
 namespace {
-
-constexpr int BM = 256;                    // rows of a macro tile
-constexpr int BN = 256;                    // columns of a macro tile
-constexpr int KBYTES = 64;                 // bytes of K per row per k-step
-constexpr int X_TILE_BYTES = BM * KBYTES;  // activation tile of one stage: 16 KiB
-constexpr int W_TILE_BYTES = BN * KBYTES;
-constexpr int STAGE_BYTES = X_TILE_BYTES + W_TILE_BYTES;
-constexpr int STAGES = 5;                  // 160 KiB: the whole LDS of a CU
-constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
-constexpr int NTHREADS = 256;
-constexpr int kMaxExperts = 1024;
-
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef int i32x4 __attribute__((ext_vector_type(4)));
-typedef int i32x8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-typedef float f32x2 __attribute__((ext_vector_type(2)));
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-
-struct GemmParams {
-  const uint8_t *a;
-  const uint8_t *b;
-  void *d;
-  const int32_t *splits;
-  const int32_t *gather_a;
-  const int32_t *scatter_d;
-  const float *alpha;
-  const float *row_scale;
-  const float *col_scale;
-  const float *scalar_dev;
-  float scalar;
-  int32_t nexperts;
-  int32_t max_rows;
-  int32_t a_rows;
-  int32_t n;
-  int32_t k;
-  int32_t d_fp32;
-};
-
-#define FLUXMI_WAITCNT(vm, lgkm) \
-  __builtin_amdgcn_s_waitcnt(((vm)&15) | (((vm) >> 4) << 14) | (7 << 4) | ((lgkm) << 8))
-
-typedef __attribute__((address_space(3))) void *lds_ptr_t;
-typedef const __attribute__((address_space(1))) void *gbl_ptr_t;
-
-// One wave-wide direct-to-LDS load: lane l fetches 16 bytes from `src` (per lane) and the hardware
-// stores them at lds_base + 16*l (lds_base is wave-uniform).
-__device__ __forceinline__ void load_to_lds16(const uint8_t *src, uint8_t *lds_base) {
-  __builtin_amdgcn_global_load_lds((gbl_ptr_t)src, (lds_ptr_t)lds_base, 16, 0, 0);
-}
-
-// Two floats to packed bf16, round to nearest even (one v_cvt_pk_bf16_f32).
-__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-  const f32x2 v = {lo, hi};
-  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
-}
-
-// Source of the ring fills of a k-step past the end of K: every lane reads 16 zero bytes.
-__device__ __attribute__((aligned(1024))) const uint8_t g_zero_page[1024] = {};
-
-// MFMA geometry per element type.  bf16 uses v_mfma_f32_16x16x32_bf16: one instruction consumes a whole
-// k-step (32 elements) of a 16-row block of each operand, i.e. one 16-byte fragment register set per
-// block, and accumulates a 16x16 block in 4 registers.  At the same FLOP rate as the 32x32x16 form it
-// moves half the accumulator bytes per FLOP through the register file, and measured under the board's
-// power limit that is worth 18 % of sustained MFMA throughput.  fp8 uses the 32x32x64 f8f6f4 form: two
-// 16-byte fragment chunks per 32-row block and k-step, 16 accumulator registers per block.
-template <int ELT>
-struct Geom {
-  static constexpr int BLK = ELT == 2 ? 16 : 32;  // rows (columns) of an operand block
-  static constexpr int NCH = ELT == 2 ? 1 : 2;    // 16-byte fragment chunks per block and k-step
-  static constexpr int NACC = BLK * BLK / 64;     // accumulator registers per block
-  typedef float Acc __attribute__((ext_vector_type(NACC)));
-};
-
-// MFMA number t of a k-step over MBK x NBK blocks: block row i = t / NBK, block column j = t % NBK.
-template <int ELT, int MBK, int NBK>
-__device__ __forceinline__ void mfma_slot(int t, const i32x4 (&xf)[MBK][Geom<ELT>::NCH], const i32x4 (&wf)[NBK][Geom<ELT>::NCH],
-                                          typename Geom<ELT>::Acc (&acc)[MBK][NBK]) {
-  const int i = t / NBK, j = t % NBK;
-  if constexpr (ELT == 2) {
-    // Written as asm to pin the accumulators to the accumulation registers: given the builtin, the
-    // register allocator spreads the 64 four-register accumulators over both register files and shuffles
-    // them at the loop's back edge.  Every accumulator is touched once per k-step, 63 MFMAs apart, and
-    // the fragment operands come from LDS reads the compiler still tracks, so no hazard needs software
-    // wait states here.
-    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(wf[j][0]), "v"(xf[i][0]));
-  } else {
-    i32x8 wa, xa;
-#pragma unroll
-    for (int v = 0; v < 4; ++v) {
-      wa[v] = wf[j][0][v];
-      wa[4 + v] = wf[j][1][v];
-      xa[v] = xf[i][0][v];
-      xa[4 + v] = xf[i][1][v];
-    }
-    // cbsz = blgp = 0: both operands e4m3; zero scale operands select the unscaled form (scale 1).
-    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wa, xa, acc[i][j], 0, 0, 0, 0, 0, 0);
-  }
-}
-
-// Clamped row count of expert e: negative entries count as 0 and rows past max_rows do not exist.
-__device__ __forceinline__ int expert_rows(const GemmParams &p, int e, int row_base) {
-  int rows = p.splits[e];
-  if (rows < 0) rows = 0;
-  if (rows > p.max_rows - row_base) rows = p.max_rows - row_base;
-  return rows;
-}
-
-// Per-lane constants shared by all tile shapes.
-struct TileCtx {
-  int wave, lane, wn, wm;
-  int fill_row, fill_chunk;
-  int frag_off[2];
-  int nk;
-  int64_t kbytes;
-  float scalar;
-};
-
-// The kernel's only argument, read again from the kernel argument segment where it is used.  A copy of
-// all of it kept live in scalar registers through the main loop does not fit the register file; the
-// empty asm keeps the compiler from hoisting these loads back to the top of the kernel.
-typedef const __attribute__((address_space(4))) GemmParams *KernArgs;
-__device__ __forceinline__ KernArgs kernel_args() {
-  KernArgs k = (KernArgs)__builtin_amdgcn_kernarg_segment_ptr();
-  asm volatile("" : "+s"(k));
-  return k;
-}
-
-// One accumulator element, moved out of its accumulation register at the point of use.  Left to itself
-// the compiler copies all 256 of them into vector registers ahead of the epilogue's branches, which
-// does not fit.
-__device__ __forceinline__ float acc_read(float a) {
-  float v;
-  asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(a));
-  return v;
-}
-
-// Epilogue of one wave: acc (32*MB rows x 32*NB columns, MFMA layout) -> scaled, cast, stored.
-// Blocks of 64 rows x 32 columns go through one of two 8 KiB LDS windows in fp32 (alternating, so the
-// writes of a block do not wait for the reads of the one before) and come back with eight lanes per
-// row (j below counts 32-column groups, ip 64-row groups).  FULL: every row and column of the wave's quarter exists and rows are stored where they are (no
-// scatter), so no store is predicated.  OUT_F32 selects the output element type.  !SCALED: every scale
-// factor is 1 and the multiplications are left out.
-template <int ELT, int MB, int NB, bool FULL, bool OUT_F32, bool SCALED>
-__device__ __forceinline__ void store_tile(uint8_t *windows, const TileCtx &c, int e, int row_base, int rows_e, int wrow0,
-                                           int wcol0,
-                                           const typename Geom<ELT>::Acc (&acc)[32 * MB / Geom<ELT>::BLK][32 * NB / Geom<ELT>::BLK]) {
-  static_assert(MB % 2 == 0, "a window holds 64 rows");
-  constexpr int BLK = Geom<ELT>::BLK;
-  constexpr int MBK = 32 * MB / BLK;
-  constexpr int ELT_OUT = OUT_F32 ? 4 : 2;
-  const KernArgs p = kernel_args();
-  const int lane = c.lane;
-  const int h = lane >> 5;
-  const int n = p->n;
-  const float *alpha = p->alpha, *row_scale = p->row_scale, *col_scale = p->col_scale;
-  const float tile_scale = c.scalar * (alpha ? alpha[e] : 1.f);
-  float rs[MBK];  // scale of this lane's row in each block row
-#pragma unroll
-  for (int i = 0; i < MBK; ++i) {
-    const int m = wrow0 + i * BLK + (lane & (BLK - 1));
-    rs[i] = tile_scale * ((row_scale && (FULL || m < rows_e)) ? row_scale[row_base + m] : 1.f);
-  }
-  const int rr0 = lane >> 3;  // row of this lane within a group of 8 rows (store phase)
-  const int cc = lane & 7;    // its 4-column chunk
-  // Output address of (first row of the wave + rr0, first column of the wave + 4 * cc); blocks and row
-  // groups add multiples of 32 columns and 8 rows.
-  uint8_t *const d = static_cast<uint8_t *>(p->d);
-  uint8_t *dlane = d + (static_cast<int64_t>(row_base + wrow0 + rr0) * n + wcol0 + cc * 4) * ELT_OUT;
-  const int64_t rowgroup_bytes = static_cast<int64_t>(8) * n * ELT_OUT;
-  const int32_t *scatter = FULL ? nullptr : p->scatter_d;
-  const int max_rows = p->max_rows;
-  int block = 0;
-#pragma unroll
-  for (int j = 0; j < NB; ++j) {
-    const int col = wcol0 + j * 32 + cc * 4;
-    float4 cs = make_float4(1.f, 1.f, 1.f, 1.f);
-    if (col_scale && (FULL || col < n)) cs = *reinterpret_cast<const float4 *>(col_scale + static_cast<int64_t>(e) * n + col);
-#pragma unroll
-    for (int ip = 0; ip < MB / 2; ++ip, ++block) {
-      uint8_t *window = windows + (block & 1) * 8192;
-      // write phase.  A lane holds one row of a block and groups of 4 consecutive columns of it: with
-      // 16x16 blocks one group, columns 4 * (lane / 16); with 32x32 blocks four, columns 8q + 4 * (lane / 32).
-#pragma unroll
-      for (int ii = 0; ii < 64 / BLK; ++ii) {
-        const int i = ip * (64 / BLK) + ii;
-        const int r = ii * BLK + (lane & (BLK - 1));
-#pragma unroll
-        for (int jj = 0; jj < 32 / BLK; ++jj) {
-          const int jb = j * (32 / BLK) + jj;
-#pragma unroll
-          for (int q = 0; q < Geom<ELT>::NACC / 4; ++q) {
-            const int chunk = BLK == 32 ? 2 * q + h : jj * 4 + (lane >> 4);
-            float4 v = make_float4(acc_read(acc[i][jb][4 * q + 0]), acc_read(acc[i][jb][4 * q + 1]),
-                                   acc_read(acc[i][jb][4 * q + 2]), acc_read(acc[i][jb][4 * q + 3]));
-            if constexpr (SCALED) v = make_float4(v.x * rs[i], v.y * rs[i], v.z * rs[i], v.w * rs[i]);
-            *reinterpret_cast<float4 *>(window + r * 128 + ((chunk ^ ((r >> 1) & 7)) << 4)) = v;
-          }
-        }
-      }
-      // store phase: 8 lanes per row, 8 rows per instruction
-      float4 v[8];
-#pragma unroll
-      for (int it = 0; it < 8; ++it) {
-        const int rr = it * 8 + rr0;
-        v[it] = *reinterpret_cast<const float4 *>(window + rr * 128 + ((cc ^ ((rr >> 1) & 7)) << 4));
-      }
-      uint8_t *dp = dlane + (static_cast<int64_t>(ip) * 8) * rowgroup_bytes + j * 32 * ELT_OUT;
-#pragma unroll
-      for (int it = 0; it < 8; ++it, dp += rowgroup_bytes) {
-        uint8_t *dst = dp;
-        if constexpr (!FULL) {
-          const int m = wrow0 + ip * 64 + it * 8 + rr0;
-          if (m >= rows_e || col >= n) continue;  // n % 4 == 0: a chunk is all in or all out
-          if (scatter) {
-            const int64_t drow = scatter[row_base + m];
-            if (drow < 0 || drow >= max_rows) continue;
-            dst = d + (drow * n + col) * ELT_OUT;
-          }
-        }
-        float4 o = v[it];
-        if constexpr (SCALED) o = make_float4(o.x * cs.x, o.y * cs.y, o.z * cs.z, o.w * cs.w);
-        if constexpr (OUT_F32) {
-          *reinterpret_cast<float4 *>(dst) = o;
-        } else {
-          u32x2 b;
-          b[0] = pack_bf16x2(o.x, o.y);
-          b[1] = pack_bf16x2(o.z, o.w);
-          *reinterpret_cast<u32x2 *>(dst) = b;
-        }
-      }
-    }
-  }
-}
-
-// Compile-time loop: f(integral_constant<int, I>) for I in [0, N).
-template <int I, int N, class F>
-__device__ __forceinline__ void static_for(F &&f) {
-  if constexpr (I < N) {
-    f(std::integral_constant<int, I>{});
-    static_for<I + 1, N>(f);
-  }
-}
-
-// Buffer resource over [base, base + bytes): loads past the end return zero instead of faulting.
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const uint8_t *base, int64_t bytes) {
-  const uint32_t n = bytes > 0xffffffffll ? 0xffffffffu : static_cast<uint32_t>(bytes < 0 ? 0 : bytes);
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(base), 0, static_cast<int>(n), 0x00020000);
-}
-
-// One output tile of (64*MB) rows x (64*NB) columns at rows [m0, ..) of expert e, columns [n0, ..).
-// (MB, NB) = (4, 4) is the macro tile, (2, 4) its upper half (for the last rows of an expert); (4, 2) and
-// (2, 2) are the 256x128 and 128x128 pieces a tile of the last, partly filled round is cut into.  Waves
-// are laid out 2 x 2.
-template <int ELT, int MB, int NB>
-__device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, const TileCtx &c, int e, int row_base,
-                                          int rows_e, int m0, int n0) {
-  constexpr int XLOADS = MB;           // direct-to-LDS instructions per wave per stage, X tile
-  constexpr int WLOADS = NB;           // same, W tile
-  constexpr int LOADS = XLOADS + WLOADS;
-  constexpr int BLK = Geom<ELT>::BLK, NCH = Geom<ELT>::NCH;
-  constexpr int MBK = 32 * MB / BLK, NBK = 32 * NB / BLK;  // operand blocks of a wave
-  constexpr int NR = (MBK + NBK) * NCH;  // fragment reads per k-step (16 bytes per lane each)
-  constexpr int NM = MBK * NBK;          // MFMAs per k-step
-  constexpr int RSPAN = NM / 2;        // MFMA slots over which the fragment reads of a step are spread
-  const int wave = c.wave, lane = c.lane, wm = c.wm, wn = c.wn, nk = c.nk;
-
-  // Ring fills address global memory through buffer resources: a scalar base per operand, a
-  // loop-invariant 32-bit byte offset per lane and fill instruction, and the k offset as scalar offset
-  // plus immediate.  Fill instruction q of a tile covers rows [16q, 16q+16); tail rows re-read the last
-  // valid row.
-  const bool gathered = p.gather_a != nullptr;
-  const uint8_t *xbase = gathered ? p.a : p.a + static_cast<int64_t>(row_base + m0) * c.kbytes;
-  const int64_t xrows = gathered ? p.a_rows : rows_e - m0;
-  const int64_t xbytes = xrows > 0 ? xrows * c.kbytes : 0xffffffffll;
-  const uint8_t *wbase = p.b + (static_cast<int64_t>(e) * p.n + n0) * c.kbytes;
-  const int64_t wbytes = static_cast<int64_t>(p.n - n0) * c.kbytes;
-  // An odd number of k-steps is rounded up by a phantom step whose fragments come from a page of zeros
-  // (every lane at offset 16 * lane).
-  const __amdgpu_buffer_rsrc_t xrsrc = make_rsrc(xbase, xbytes);
-  const __amdgpu_buffer_rsrc_t wrsrc = make_rsrc(wbase, wbytes);
-  const __amdgpu_buffer_rsrc_t zrsrc = make_rsrc(g_zero_page, 1024);
-  const uint32_t zoff = lane * 16;
-  uint32_t xoff[XLOADS], woff[WLOADS];
-#pragma unroll
-  for (int j = 0; j < XLOADS; ++j) {
-    int xr = m0 + (XLOADS * wave + j) * 16 + c.fill_row;
-    if (xr > rows_e - 1) xr = rows_e - 1;
-    int64_t arow = xr - m0;
-    if (gathered) {
-      arow = p.gather_a[row_base + xr];
-      if (p.a_rows > 0) arow = arow < 0 ? 0 : (arow >= p.a_rows ? p.a_rows - 1 : arow);
-    }
-    xoff[j] = static_cast<uint32_t>(arow * c.kbytes) + c.fill_chunk * 16;
-  }
-#pragma unroll
-  for (int j = 0; j < WLOADS; ++j) {
-    int wr = n0 + (WLOADS * wave + j) * 16 + c.fill_row;
-    if (wr > p.n - 1) wr = p.n - 1;
-    woff[j] = static_cast<uint32_t>((wr - n0) * c.kbytes) + c.fill_chunk * 16;
-  }
-  // LDS destinations of this wave's fill instructions inside a stage (X rows first, then W rows).
-  uint8_t *xdst = smem + (XLOADS * wave) * 1024;
-  uint8_t *wdst = smem + X_TILE_BYTES + (WLOADS * wave) * 1024;
-
-  // Fill instruction Q of the k-step at byte offset kbyte of every row, into ring slot SLOT (compile-time
-  // slot: the LDS address is an immediate).  The k offset travels as the scalar offset: an instruction
-  // immediate would also be added to the LDS address.
-  auto fill_one = [&](auto SLOT, auto Q, int kbyte) {
-    constexpr int slot = decltype(SLOT)::value, q = decltype(Q)::value;
-    if constexpr (q < XLOADS)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(xrsrc, (lds_ptr_t)(xdst + slot * STAGE_BYTES + q * 1024), 16,
-                                               static_cast<int>(xoff[q]), kbyte, 0, 0);
-    else
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(wrsrc, (lds_ptr_t)(wdst + slot * STAGE_BYTES + (q - XLOADS) * 1024), 16,
-                                               static_cast<int>(woff[q - XLOADS]), kbyte, 0, 0);
-  };
-  // Same with a run-time slot, for the last steps of a tile; a k-step past the end of K (the phantom
-  // second half of the last pair of an odd K) is filled from the zero page.
-  auto fill_dyn = [&](int slot, auto Q, int kstep) {
-    constexpr int q = decltype(Q)::value;
-    const bool in = kstep < nk;
-    const int kbyte = in ? kstep * KBYTES : 0;
-    if constexpr (q < XLOADS)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(in ? xrsrc : zrsrc, (lds_ptr_t)(xdst + slot * STAGE_BYTES + q * 1024), 16,
-                                               static_cast<int>(in ? xoff[q] : zoff), kbyte, 0, 0);
-    else
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(in ? wrsrc : zrsrc, (lds_ptr_t)(wdst + slot * STAGE_BYTES + (q - XLOADS) * 1024),
-                                               16, static_cast<int>(in ? woff[q - XLOADS] : zoff), kbyte, 0, 0);
-  };
-
-  typename Geom<ELT>::Acc acc[MBK][NBK];
-#pragma unroll
-  for (int i = 0; i < MBK; ++i)
-#pragma unroll
-    for (int j = 0; j < NBK; ++j)
-#pragma unroll
-      for (int v = 0; v < Geom<ELT>::NACC; ++v) acc[i][j][v] = 0.f;
-
-  // Fragment addresses: per lane and 16-byte chunk s a base for each operand; a stage and block add a
-  // compile-time offset.  LDS instructions carry 16 bits of offset, so three bases 64 KiB apart.
-  const uint8_t *xfrag[3][NCH], *wfrag[3][NCH];
-#pragma unroll
-  for (int hi = 0; hi < 3; ++hi)
-#pragma unroll
-    for (int s = 0; s < NCH; ++s) {
-      xfrag[hi][s] = smem + hi * 65536 + wm * (32 * MB) * KBYTES + c.frag_off[s];
-      wfrag[hi][s] = smem + hi * 65536 + X_TILE_BYTES + wn * (32 * NB) * KBYTES + c.frag_off[s];
-    }
-  i32x4 xa[MBK][NCH], wa[NBK][NCH], xb[MBK][NCH], wb[NBK][NCH];
-  // Fragment read R of the k-step in ring slot SLOT: chunk s = R / (MBK + NBK) of W block q (q < NBK) or of
-  // X block q - NBK.
-  auto read_one = [&](auto SLOT, auto R, i32x4 (&xf)[MBK][NCH], i32x4 (&wf)[NBK][NCH]) {
-    constexpr int slot = decltype(SLOT)::value, r = decltype(R)::value;
-    constexpr int s = r / (MBK + NBK), q = r % (MBK + NBK);
-    constexpr int hi = (slot * STAGE_BYTES) / 65536, lo = (slot * STAGE_BYTES) % 65536;
-    if constexpr (q < NBK) wf[q][s] = *reinterpret_cast<const i32x4 *>(wfrag[hi][s] + lo + q * BLK * KBYTES);
-    else xf[q - NBK][s] = *reinterpret_cast<const i32x4 *>(xfrag[hi][s] + lo + (q - NBK) * BLK * KBYTES);
-  };
-
-  auto read_dyn = [&](int slot, auto R, i32x4 (&xf)[MBK][NCH], i32x4 (&wf)[NBK][NCH]) {
-    constexpr int r = decltype(R)::value;
-    constexpr int s = r / (MBK + NBK), q = r % (MBK + NBK);
-    if constexpr (q < NBK) wf[q][s] = *reinterpret_cast<const i32x4 *>(wfrag[0][s] + slot * STAGE_BYTES + q * BLK * KBYTES);
-    else xf[q - NBK][s] = *reinterpret_cast<const i32x4 *>(xfrag[0][s] + slot * STAGE_BYTES + (q - NBK) * BLK * KBYTES);
-  };
-
-  // One k-step, number U within a run of ten (ring of five slots x two fragment sets: after ten steps
-  // every slot index and register role repeats, so all of them are compile-time constants here).
-  // MFMAs run on `cur` (read during the previous step), the fragments of the next step go into `nxt`,
-  // and half of the fills of the pair of steps (E+4, E+5), E = U rounded down to even, are issued:
-  // that pair is requested over the two steps E and E+1, row group by row group, both k-steps of a row
-  // group back to back (the second one hits the line the first one brought into L1).
-  auto step = [&](auto U, int kbase, i32x4 (&xc)[MBK][NCH], i32x4 (&wc)[NBK][NCH], i32x4 (&xn)[MBK][NCH], i32x4 (&wn_)[NBK][NCH]) {
-    constexpr int u = decltype(U)::value;
-    constexpr bool even = (u & 1) == 0;
-    constexpr int e0 = u & ~1;
-    // Stage u+1 has landed once the pair it belongs to is complete; fills are counted in issue order.
-    if constexpr (even) {
-      FLUXMI_WAITCNT(2 * LOADS, 15);  // all but the pair requested during the last two steps
-    } else {
-      FLUXMI_WAITCNT(LOADS, 15);      // all but the half pair requested during the last step
-    }
-    __builtin_amdgcn_s_barrier();     // ... for every wave's share; and everybody is done reading stage u
-    __builtin_amdgcn_sched_barrier(0);
-    static_for<0, NM>([&](auto T) {
-      constexpr int t = decltype(T)::value;
-      static_for<0, NR>([&](auto R) {
-        constexpr int r = decltype(R)::value;
-        if constexpr (r * RSPAN / NR == t) read_one(std::integral_constant<int, (u + 1) % STAGES>{}, R, xn, wn_);
-      });
-      static_for<0, 2 * LOADS>([&](auto D) {
-        constexpr int d = decltype(D)::value;
-        if constexpr ((d * (2 * NM) / (2 * LOADS) + 1) % (2 * NM) == t + (even ? 0 : NM))
-          fill_one(std::integral_constant<int, (e0 + 4 + (d & 1)) % STAGES>{}, std::integral_constant<int, (d >> 1)>{},
-                   kbase + (e0 + 4 + (d & 1)) * KBYTES);
-      });
-      mfma_slot<ELT, MBK, NBK>(t, xc, wc, acc);
-      __builtin_amdgcn_sched_barrier(0);
-    });
-    FLUXMI_WAITCNT(63, 0);  // the fragments of the next step are in registers (requested long ago)
-    __builtin_amdgcn_sched_barrier(0);
-  };
-  // The same step with run-time ring slots (k-step ks, slot ks % 5), for the last steps of a tile, whose
-  // number is not a multiple of ten.
-  auto step_dyn = [&](int ks, bool even, i32x4 (&xc)[MBK][NCH], i32x4 (&wc)[NBK][NCH], i32x4 (&xn)[MBK][NCH], i32x4 (&wn_)[NBK][NCH]) {
-    if (even) {
-      FLUXMI_WAITCNT(2 * LOADS, 15);
-    } else {
-      FLUXMI_WAITCNT(LOADS, 15);
-    }
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_sched_barrier(0);
-    const int e0 = even ? ks : ks - 1;
-    const int rslot = (ks + 1) % STAGES, pslot0 = (e0 + 4) % STAGES, pslot1 = (e0 + 5) % STAGES;
-    static_for<0, NM>([&](auto T) {
-      constexpr int t = decltype(T)::value;
-      static_for<0, NR>([&](auto R) {
-        constexpr int r = decltype(R)::value;
-        if constexpr (r * RSPAN / NR == t) read_dyn(rslot, R, xn, wn_);
-      });
-      static_for<0, 2 * LOADS>([&](auto D) {
-        constexpr int d = decltype(D)::value;
-        constexpr int at = (d * (2 * NM) / (2 * LOADS) + 1) % (2 * NM);
-        if constexpr (at < NM) {
-          if (at == t && even) fill_dyn((d & 1) ? pslot1 : pslot0, std::integral_constant<int, (d >> 1)>{}, e0 + 4 + (d & 1));
-        } else {
-          if (at - NM == t && !even) fill_dyn((d & 1) ? pslot1 : pslot0, std::integral_constant<int, (d >> 1)>{}, e0 + 4 + (d & 1));
-        }
-      });
-      mfma_slot<ELT, MBK, NBK>(t, xc, wc, acc);
-      __builtin_amdgcn_sched_barrier(0);
-    });
-    FLUXMI_WAITCNT(63, 0);
-    __builtin_amdgcn_sched_barrier(0);
-  };
-
-  // ---- prologue: request k-steps 0..3 as two pairs, wait for the first pair ------------------------
-  FLUXMI_WAITCNT(0, 0);  // stores of the previous tile's epilogue
-  static_for<0, 2>([&](auto P) {
-    constexpr int s = 2 * decltype(P)::value;
-    static_for<0, LOADS>([&](auto Q) {
-      fill_dyn(s, Q, s);
-      fill_dyn(s + 1, Q, s + 1);
-    });
-  });
-  FLUXMI_WAITCNT(2 * LOADS, 15);
-  __builtin_amdgcn_s_barrier();
-  static_for<0, NR>([&](auto R) { read_one(std::integral_constant<int, 0>{}, R, xa, wa); });
-  FLUXMI_WAITCNT(63, 0);  // in registers before the first step's barrier lets anyone refill that slot
-
-  // ---- main loop ----------------------------------------------------------------------------------
-  // Whole trips of ten k-steps while every k-step a trip requests (up to 13 past its first one) exists,
-  // then the remaining 4 to 23 steps pair by pair with run-time ring slots.  An odd number of k-steps
-  // ends with a phantom step on zero fragments.
-  const int nfast = nk >= 14 ? (nk - 14) / 10 + 1 : 0;  // trips with 10 * trip + 13 < nk
-  int kbase = 0;  // byte offset along K of step 0 of the current trip
-  for (int trip = 0; trip < nfast; ++trip) {
-    step(std::integral_constant<int, 0>{}, kbase, xa, wa, xb, wb);
-    step(std::integral_constant<int, 1>{}, kbase, xb, wb, xa, wa);
-    step(std::integral_constant<int, 2>{}, kbase, xa, wa, xb, wb);
-    step(std::integral_constant<int, 3>{}, kbase, xb, wb, xa, wa);
-    step(std::integral_constant<int, 4>{}, kbase, xa, wa, xb, wb);
-    step(std::integral_constant<int, 5>{}, kbase, xb, wb, xa, wa);
-    step(std::integral_constant<int, 6>{}, kbase, xa, wa, xb, wb);
-    step(std::integral_constant<int, 7>{}, kbase, xb, wb, xa, wa);
-    step(std::integral_constant<int, 8>{}, kbase, xa, wa, xb, wb);
-    step(std::integral_constant<int, 9>{}, kbase, xb, wb, xa, wa);
-    kbase += 10 * KBYTES;
-  }
-  for (int ks = 10 * nfast; ks < nk; ks += 2) {
-    step_dyn(ks, true, xa, wa, xb, wb);
-    step_dyn(ks + 1, false, xb, wb, xa, wa);
-  }
-
-  // ---- epilogue ---------------------------------------------------------------------------------
-  FLUXMI_WAITCNT(0, 0);          // this wave's trailing ring fills have landed
-  __builtin_amdgcn_s_barrier();  // ... and everybody else's; nobody reads the ring any more
-  uint8_t *windows = smem + wave * 16384;  // two 8 KiB windows per wave
-  const int wrow0 = m0 + wm * (32 * MB);
-  const int wcol0 = n0 + wn * (32 * NB);
-  {
-    const KernArgs pe = kernel_args();
-    const bool full = wrow0 + 32 * MB <= rows_e && wcol0 + 32 * NB <= pe->n && pe->scatter_d == nullptr;
-    const bool out_f32 = pe->d_fp32 != 0;
-    const bool scaled = !(c.scalar == 1.f && pe->alpha == nullptr && pe->row_scale == nullptr && pe->col_scale == nullptr);
-    if (full && !scaled) {
-      if (out_f32) store_tile<ELT, MB, NB, true, true, false>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
-      else store_tile<ELT, MB, NB, true, false, false>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
-    } else if (full) {
-      if (out_f32) store_tile<ELT, MB, NB, true, true, true>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
-      else store_tile<ELT, MB, NB, true, false, true>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
-    } else {
-      if (out_f32) store_tile<ELT, MB, NB, false, true, true>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
-      else store_tile<ELT, MB, NB, false, false, true>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
-    }
-  }
-  __builtin_amdgcn_s_barrier();  // the LDS windows are free again before the next tile's fills start
-}
-
-template <int ELT>
-__global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmParams p) {
-  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];  // STAGES x (X tile | W tile)
-
-  TileCtx c;
-  const int tid = threadIdx.x;
-  c.wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: branches on it stay uniform
-  c.lane = tid & 63;
-  c.wn = c.wave & 1;   // column half
-  c.wm = c.wave >> 1;  // row half
-  const int lane = c.lane;
-  const int tiles_n = (p.n + BN - 1) / BN;
-  c.kbytes = static_cast<int64_t>(p.k) * ELT;
-  c.nk = static_cast<int>(c.kbytes / KBYTES);
-
-  // LDS tile layout: rows of 64 bytes, four rows per 256-byte "superline" S = r >> 2 (the LDS serves
-  // 64 banks x 4 bytes per clock, 16 lanes of a 16-byte read at a time).  (row r, chunk c) sits in
-  // 16-byte slot ((r & 3) << 2) | (c ^ (S & 3)) of its superline, so the 16 rows read together by a
-  // quarter wave (same chunk) fall into 16 different slots.
-  // Direct-to-LDS fill: instruction q of a tile covers rows [16q, 16q+16) = 1 KiB; lane l lands in
-  // superline 4q + (l >> 4), slot l & 15, i.e. row 16q + (l >> 2), chunk (l & 3) ^ ((l >> 4) & 3).
-  c.fill_row = lane >> 2;
-  c.fill_chunk = (lane & 3) ^ ((lane >> 4) & 3);
-  // Fragment reads.  bf16: lane l reads row (l & 15) of a 16-row block, chunk l >> 4 (the four chunks of
-  // a row are the 32 k-elements of one MFMA).  fp8: row (l & 31) of a 32-row block, chunks 2 * (l >> 5) + s.
-  if (ELT == 2) {
-    const int r = lane & 15, ch = lane >> 4;
-    const int slot = ((r & 3) << 2) | (ch ^ ((r >> 2) & 3));
-    c.frag_off[0] = (r >> 2) * 256 + slot * 16;
-    c.frag_off[1] = 0;
-  } else {
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      const int ch = 2 * (lane >> 5) + s;
-      const int slot = ((lane & 3) << 2) | (ch ^ ((lane >> 2) & 3));
-      c.frag_off[s] = ((lane & 31) >> 2) * 256 + slot * 16;
-    }
-  }
-  c.scalar = p.scalar;
-  if (p.scalar_dev) c.scalar *= p.scalar_dev[0];
-
-  const int grid = gridDim.x;
-  const int bid = blockIdx.x;
-  // Workgroups are dealt to XCDs round-robin; give each XCD a run of consecutive logical work items.
-  const int virt = (grid % 8 == 0) ? (bid & 7) * (grid >> 3) + (bid >> 3) : bid;
-
-  // ---- total tile count (one wave-wide pass over splits) -> shape of the last round -----------------
-  int total_tiles = 0;
-  {
-    int row_carry = 0, acc_tiles = 0;
-    for (int e0 = 0; e0 < p.nexperts; e0 += 64) {
-      const int ee = e0 + lane;
-      int rows = ee < p.nexperts ? p.splits[ee] : 0;
-      if (rows < 0) rows = 0;
-      const int incl = wave_inclusive_scan(rows);
-      int begin = row_carry + incl - rows, end = row_carry + incl;
-      if (begin > p.max_rows) begin = p.max_rows;
-      if (end > p.max_rows) end = p.max_rows;
-      int tiles = ((end - begin + BM - 1) / BM) * tiles_n;
-#pragma unroll
-      for (int off = 32; off > 0; off >>= 1) tiles += __shfl_xor(tiles, off, 64);
-      acc_tiles += tiles;
-      row_carry += __shfl(incl, 63, 64);
-    }
-    total_tiles = __builtin_amdgcn_readfirstlane(acc_tiles);
-  }
-  // Full rounds run whole macro tiles.  The tiles of the last, partly filled round are cut into
-  // `pieces` parts (2 pieces of 256x128, or 4 of 128x128) when that still fits one round, so that the
-  // chip does not idle while a fraction of the CUs finishes whole tiles.
-  const int full_items = (total_tiles / grid) * grid;
-  const int rem_tiles = total_tiles - full_items;
-  const int pieces = rem_tiles * 4 <= grid ? 4 : (rem_tiles * 2 <= grid ? 2 : 1);
-  const int total_items = full_items + rem_tiles * pieces;
-
-  // ---- schedule: walk the experts once, in step with this workgroup's increasing tile ids ----------
-  // All of it is wave-uniform scalar work on the device-resident splits (no LDS, no host round trip).
-  int e = 0;
-  int row_base = 0;   // sorted rows before expert e
-  int tile_base = 0;  // tiles before expert e
-  int rows_e = expert_rows(p, 0, 0);
-  int tiles_e = ((rows_e + BM - 1) / BM) * tiles_n;
-
-  for (int item = virt; item < total_items; item += grid) {
-    int tile = item, piece = 0;
-    if (item >= full_items) {
-      tile = full_items + (item - full_items) / pieces;
-      piece = (item - full_items) % pieces;
-    }
-    while (e < p.nexperts && tile >= tile_base + tiles_e) {
-      tile_base += tiles_e;
-      row_base += rows_e;
-      ++e;
-      if (e < p.nexperts) {
-        rows_e = expert_rows(p, e, row_base);
-        tiles_e = ((rows_e + BM - 1) / BM) * tiles_n;
-      }
-    }
-    if (e >= p.nexperts) break;
-    // Order inside an expert: row tiles are cut into groups of at most 8; a group is walked
-    // column-major over all weight panels before the next group starts.  32 consecutive tiles (one
-    // XCD's share of a round) then cover about 8 row tiles x 4 panels: 12 distinct operand tiles per
-    // k-step for 32 CUs.
-    const int m_tiles = (rows_e + BM - 1) / BM;
-    const int ngroups_m = (m_tiles + 7) >> 3;
-    const int gm = (m_tiles + ngroups_m - 1) / ngroups_m;  // group height, <= 8
-    const int local = tile - tile_base;
-    const int group = local / (gm * tiles_n);
-    const int group_first = group * gm;
-    const int group_rows = m_tiles - group_first < gm ? m_tiles - group_first : gm;
-    const int in_group = local - group * gm * tiles_n;
-    const int nt = in_group / group_rows;
-    const int mt = group_first + (in_group - nt * group_rows);
-    int m0 = mt * BM;
-    int n0 = nt * BN;
-
-    if (item < full_items || pieces == 1) {
-      // The last row tile of an expert is run 128 rows high when that covers its rows.
-      if (rows_e - m0 > 128) gemm_tile<ELT, 4, 4>(p, smem, c, e, row_base, rows_e, m0, n0);
-      else gemm_tile<ELT, 2, 4>(p, smem, c, e, row_base, rows_e, m0, n0);
-    } else if (pieces == 2) {
-      n0 += piece * 128;
-      if (n0 < p.n) gemm_tile<ELT, 4, 2>(p, smem, c, e, row_base, rows_e, m0, n0);
-    } else {
-      m0 += (piece >> 1) * 128;
-      n0 += (piece & 1) * 128;
-      if (m0 < rows_e && n0 < p.n) gemm_tile<ELT, 2, 2>(p, smem, c, e, row_base, rows_e, m0, n0);
-    }
-  }
-}
 
 // ---- generic kernel: any K / N, no alignment demands beyond element size -------------------------
 // One thread per output element, a wave covers 64 consecutive columns of one row.  Only used when the
@@ -742,15 +84,6 @@ bool mfma_path_ok(const fluxmi_grouped_gemm_args *a) {
          (a->col_scale == nullptr || aligned16(a->col_scale)) && a_fits && a->n * kbytes <= span;
 }
 
-template <int ELT>
-int launch_mfma(const GemmParams &p, int grid, hipStream_t s) {
-  static std::atomic<uint64_t> lds_done{0};
-  const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(grouped_gemm_mfma_kernel<ELT>), LDS_BYTES, lds_done);
-  if (rc != FLUXMI_OK) return rc;
-  hipLaunchKernelGGL((grouped_gemm_mfma_kernel<ELT>), dim3(grid), dim3(NTHREADS), LDS_BYTES, s, p);
-  return FLUXMI_OK;
-}
-
 }  // namespace
 }  // namespace fluxmi
 
@@ -802,7 +135,7 @@ extern "C" int fluxmi_grouped_gemm(const fluxmi_grouped_gemm_args *args, void *,
     const int64_t tiles_n = (args->n + BN - 1) / BN;
     const int64_t max_tiles = (static_cast<int64_t>(args->max_rows) / BM + args->nexperts) * tiles_n;
     const int grid = static_cast<int>(max_tiles < cus ? max_tiles : cus);
-    const int rc = args->dtype == FLUXMI_BF16 ? launch_mfma<2>(p, grid, s) : launch_mfma<1>(p, grid, s);
+    const int rc = args->dtype == FLUXMI_BF16 ? launch_grouped_gemm_bf16(p, grid, s) : launch_grouped_gemm_fp8(p, grid, s);
     if (rc != FLUXMI_OK) return rc;
   } else {
     const int grid = cus * 8;

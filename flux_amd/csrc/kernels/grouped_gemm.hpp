@@ -1,0 +1,82 @@
+// Grouped GEMM over ragged per-expert row counts: D[r,:] = scale(r,:) * A[gather(r),:] @ B[e(r)]^T.
+//
+// Persistent kernel, one 256-thread workgroup (4 waves, one per SIMD) per CU, macro tile 256 rows x 256
+// columns, k-step of 64 bytes per row (32 bf16 or 64 fp8).  Both operand tiles are staged in LDS by
+// direct-to-LDS global loads (no register staging) in a ring of five 32 KiB stages; the row gather of A
+// is folded into the per-lane global address of those loads.  Each wave owns a 128 x 128 quarter of the
+// macro tile (4x4 MFMA blocks of 32x32, 256 fp32 accumulator registers) and runs a software pipeline
+// of its own: while the MFMAs of k-step s run on one set of fragment registers, the fragments of step
+// s+1 are read from LDS into a second set and the ring fills of steps s+4 / s+5 are issued, all in a
+// fixed interleaving (one fragment read per MFMA over the first half of the step, one fill every
+// fourth MFMA).  One workgroup barrier per k-step publishes the landed stage.
+//
+// Ring fills are issued in pairs of k-steps: the two 64-byte halves of a 128-byte line are requested
+// back to back (they go to different stages), so the second request hits the line the first one
+// brought into the vector L1 and L2 sees one request per line instead of two.
+//
+// The MFMA "A" operand is the weight fragment and the "B" operand the activation fragment, i.e. the
+// hardware computes D^T blocks: a lane then holds, for one output row, four consecutive output columns
+// per accumulator quad.  The epilogue passes each 64-row x 32-column block through a wave-private LDS
+// window in fp32 and reads it back with eight lanes per row, so that one store instruction writes 64
+// (bf16) or 128 (fp32) contiguous bytes of each row.
+//
+// Tile schedule: every wave walks the device-resident `splits` with scalar loads, in step with the
+// increasing logical tile ids of its workgroup; ids are assigned so that the workgroups of one XCD
+// (those with equal blockIdx % 8) take a run of consecutive tiles; tiles of an expert are ordered in
+// groups of at most 8 row tiles, each group walked column-major over the weight panels, so an XCD's L2
+// sees a few weight panels shared by the row tiles of a group.
+#pragma once
+
+#include <cstdlib>
+#include <type_traits>
+
+#include "common.hpp"
+
+namespace fluxmi {
+
+
+constexpr int BM = 256;                    // rows of a macro tile
+constexpr int BN = 256;                    // columns of a macro tile
+constexpr int KBYTES = 64;                 // bytes of K per row per k-step
+constexpr int X_TILE_BYTES = BM * KBYTES;  // activation tile of one stage: 16 KiB
+constexpr int W_TILE_BYTES = BN * KBYTES;
+constexpr int STAGE_BYTES = X_TILE_BYTES + W_TILE_BYTES;
+constexpr int STAGES = 5;                  // 160 KiB: the whole LDS of a CU
+constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
+constexpr int NTHREADS = 256;
+constexpr int kMaxExperts = 1024;
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+struct GemmParams {
+  const uint8_t *a;
+  const uint8_t *b;
+  void *d;
+  const int32_t *splits;
+  const int32_t *gather_a;
+  const int32_t *scatter_d;
+  const float *alpha;
+  const float *row_scale;
+  const float *col_scale;
+  const float *scalar_dev;
+  float scalar;
+  int32_t nexperts;
+  int32_t max_rows;
+  int32_t a_rows;
+  int32_t n;
+  int32_t k;
+  int32_t d_fp32;
+};
+
+
+// One launcher per element type, each in a translation unit of its own (the kernel is a long compile).
+int launch_grouped_gemm_bf16(const GemmParams &p, int grid, hipStream_t s);
+int launch_grouped_gemm_fp8(const GemmParams &p, int grid, hipStream_t s);
+
+}  // namespace fluxmi

@@ -1,0 +1,6 @@
+// bf16 instantiation of the grouped GEMM MFMA kernel.
+#include "grouped_gemm_kernel.hpp"
+
+namespace fluxmi {
+int launch_grouped_gemm_bf16(const GemmParams &p, int grid, hipStream_t s) { return launch_mfma<2>(p, grid, s); }
+}  // namespace fluxmi

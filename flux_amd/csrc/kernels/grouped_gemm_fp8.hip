@@ -1,0 +1,6 @@
+// fp8 (e4m3) instantiation of the grouped GEMM MFMA kernel.
+#include "grouped_gemm_kernel.hpp"
+
+namespace fluxmi {
+int launch_grouped_gemm_fp8(const GemmParams &p, int grid, hipStream_t s) { return launch_mfma<1>(p, grid, s); }
+}  // namespace fluxmi
