@@ -106,6 +106,25 @@ def test_single_expert_matches_dense_gemm():
     assert_close(out, ref, "dense")
 
 
+@pytest.mark.parametrize("k", [96, 160, 416, 448, 480, 736, 768, 800, 1312])
+def test_bf16_k_loop_boundaries(k):
+    """K lengths around the seams of the k loop: odd numbers of 64-byte k-steps (a phantom step on zeros), the
+    hand-over from the unrolled trips of ten to the pair-wise tail (14 and 24 k-steps) and lengths on either
+    side; rows chosen so that full tiles, a 128-row tile and last-round pieces all occur."""
+    from flux_amd import capi
+    print(f"[case] grouped_gemm bf16 k-loop seams K={k}", flush=True)
+    g = torch.Generator().manual_seed(k)
+    split = np.array([300, 0, 129, 520, 77], dtype=np.int32)
+    rows, n = int(split.sum()), 520
+    a = torch.randn(rows, k, generator=g).to(torch.bfloat16)
+    w = (torch.randn(len(split), n, k, generator=g) * 0.05).to(torch.bfloat16)
+    ref = layers.grouped_gemm_fp32(a, w, split)
+    out = capi.grouped_gemm(a.cuda(), w.cuda(), torch.from_numpy(split).cuda())
+    assert_close(out, ref, f"K={k}")
+    out32 = capi.grouped_gemm(a.cuda(), w.cuda(), torch.from_numpy(split).cuda(), out_dtype=torch.float32)
+    assert torch.allclose(out32.cpu(), ref, rtol=1e-4, atol=1e-3), float((out32.cpu() - ref).abs().max())
+
+
 def sampled_rows(split, per_expert, rng):
     off = routing.offsets(split)
     rows = []
@@ -174,7 +193,7 @@ def quantise(t_bf16):
 
 
 @pytest.mark.parametrize("experts,rows,n,k,seed", [(1, 256, 256, 64, 0), (4, 1000, 512, 256, 1), (8, 2000, 1024, 1024, 2),
-                                                   (3, 300, 264, 2048, 3), (2, 40, 8, 100, 4)])
+                                                   (3, 300, 264, 2048, 3), (2, 40, 8, 100, 4), (3, 700, 264, 192, 5), (2, 300, 512, 960, 6), (4, 1100, 384, 1536, 7)])
 def test_fp8_against_dequant_matmul(experts, rows, n, k, seed):
     from flux_amd import capi
     print(f"[case] grouped_gemm fp8 E={experts} rows={rows} N={n} K={k}", flush=True)
