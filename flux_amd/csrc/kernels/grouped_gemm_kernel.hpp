@@ -147,7 +147,7 @@ __device__ __forceinline__ void store_tile(uint8_t *windows, const TileCtx &c, i
     if (col_scale && (FULL || col < n)) cs = *reinterpret_cast<const float4 *>(col_scale + static_cast<int64_t>(e) * n + col);
 #pragma unroll
     for (int ip = 0; ip < MB / 2; ++ip, ++block) {
-      uint8_t *window = windows + (block & 1) * 8192;
+      uint8_t *window = windows;
       // write phase.  A lane holds one row of a block and groups of 4 consecutive columns of it: with
       // 16x16 blocks one group, columns 4 * (lane / 16); with 32x32 blocks four, columns 8q + 4 * (lane / 32).
 #pragma unroll
@@ -217,13 +217,97 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const uint8_t *base,
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(base), 0, static_cast<int>(n), 0x00020000);
 }
 
+// Where a work item lies.  kind: 0 a whole macro tile (4, 4); 1 the 128-row tile ending an expert (2, 4);
+// 2 a 256x128 piece (4, 2); 3 a 128x128 piece (2, 2); -1 an item without work; -2 past the last item.
+struct TileDesc {
+  int kind, e, row_base, rows_e, m0, n0;
+};
+
+// Operand addressing of a tile: buffer resources and this lane's byte offsets of its fill instructions.
+template <int XL, int WL>
+struct TileOperands {
+  __amdgpu_buffer_rsrc_t xrsrc, wrsrc;
+  uint32_t xoff[XL], woff[WL];
+};
+
+// What a tile leaves behind for the next one when that is a whole macro tile: its operand addressing,
+// with k-steps 0..3 already requested into ring slots 0..3 ahead of the epilogue, so that their latency
+// passes while the epilogue runs.
+struct TilePrefetch {
+  bool valid;
+  TileOperands<4, 4> op;
+};
+
+// Ring fills address global memory through buffer resources: a scalar base per operand, a loop-invariant
+// 32-bit byte offset per lane and fill instruction, and the k offset as scalar offset.  Fill
+// instruction q of a tile covers rows [16q, 16q+16); tail rows re-read the last valid row.
+template <int XL, int WL>
+__device__ __forceinline__ void setup_operands(const GemmParams &p, const TileCtx &c, const TileDesc &t,
+                                               TileOperands<XL, WL> &op) {
+  const bool gathered = p.gather_a != nullptr;
+  const uint8_t *xbase = gathered ? p.a : p.a + static_cast<int64_t>(t.row_base + t.m0) * c.kbytes;
+  const int64_t xrows = gathered ? p.a_rows : t.rows_e - t.m0;
+  op.xrsrc = make_rsrc(xbase, xrows > 0 ? xrows * c.kbytes : 0xffffffffll);
+  op.wrsrc = make_rsrc(p.b + (static_cast<int64_t>(t.e) * p.n + t.n0) * c.kbytes, static_cast<int64_t>(p.n - t.n0) * c.kbytes);
+#pragma unroll
+  for (int j = 0; j < XL; ++j) {
+    int xr = t.m0 + (XL * c.wave + j) * 16 + c.fill_row;
+    if (xr > t.rows_e - 1) xr = t.rows_e - 1;
+    int64_t arow = xr - t.m0;
+    if (gathered) {
+      arow = p.gather_a[t.row_base + xr];
+      if (p.a_rows > 0) arow = arow < 0 ? 0 : (arow >= p.a_rows ? p.a_rows - 1 : arow);
+    }
+    op.xoff[j] = static_cast<uint32_t>(arow * c.kbytes) + c.fill_chunk * 16;
+  }
+#pragma unroll
+  for (int j = 0; j < WL; ++j) {
+    int wr = t.n0 + (WL * c.wave + j) * 16 + c.fill_row;
+    if (wr > p.n - 1) wr = p.n - 1;
+    op.woff[j] = static_cast<uint32_t>((wr - t.n0) * c.kbytes) + c.fill_chunk * 16;
+  }
+}
+
+// Fill instruction q (X rows first, then W rows) of k-step `kstep` of a tile into ring slot `slot`.  A
+// k-step past the end of K (the phantom second half of the last pair of an odd K) is filled from the
+// zero page.  The k offset travels as the scalar offset: an instruction immediate would also be added
+// to the LDS address.
+template <int XL, int WL>
+__device__ __forceinline__ void fill_any(const TileOperands<XL, WL> &op, uint8_t *smem, const TileCtx &c, int q, int slot,
+                                         int kstep) {
+  const bool in = kstep < c.nk;
+  const int kbyte = in ? kstep * KBYTES : 0;
+  const __amdgpu_buffer_rsrc_t zrsrc = make_rsrc(g_zero_page, 1024);
+  const uint32_t zoff = c.lane * 16;
+  if (q < XL)
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(in ? op.xrsrc : zrsrc, (lds_ptr_t)(smem + slot * STAGE_BYTES + (XL * c.wave + q) * 1024), 16,
+                                             static_cast<int>(in ? op.xoff[q < XL ? q : 0] : zoff), kbyte, 0, 0);
+  else
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(in ? op.wrsrc : zrsrc,
+                                             (lds_ptr_t)(smem + slot * STAGE_BYTES + X_TILE_BYTES + (WL * c.wave + (q - XL)) * 1024), 16,
+                                             static_cast<int>(in ? op.woff[q >= XL ? q - XL : 0] : zoff), kbyte, 0, 0);
+}
+
+// Requests k-steps 0..3 of a tile as two pairs into ring slots 0..3 (q is a constant after unrolling).
+template <int XL, int WL>
+__device__ __forceinline__ void issue_first_pairs(const TileOperands<XL, WL> &op, uint8_t *smem, const TileCtx &c) {
+#pragma unroll
+  for (int s = 0; s < 4; s += 2) {
+#pragma unroll
+    for (int q = 0; q < XL + WL; ++q) {
+      fill_any<XL, WL>(op, smem, c, q, s, s);
+      fill_any<XL, WL>(op, smem, c, q, s + 1, s + 1);
+    }
+  }
+}
+
 // One output tile of (64*MB) rows x (64*NB) columns at rows [m0, ..) of expert e, columns [n0, ..).
 // (MB, NB) = (4, 4) is the macro tile, (2, 4) its upper half (for the last rows of an expert); (4, 2) and
 // (2, 2) are the 256x128 and 128x128 pieces a tile of the last, partly filled round is cut into.  Waves
 // are laid out 2 x 2.
 template <int ELT, int MB, int NB>
-__device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, const TileCtx &c, int e, int row_base,
-                                          int rows_e, int m0, int n0) {
+__device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, const TileCtx &c, const TileDesc &t,
+                                          const TileDesc &next, TilePrefetch &pf) {
   constexpr int XLOADS = MB;           // direct-to-LDS instructions per wave per stage, X tile
   constexpr int WLOADS = NB;           // same, W tile
   constexpr int LOADS = XLOADS + WLOADS;
@@ -233,41 +317,26 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
   constexpr int NM = MBK * NBK;          // MFMAs per k-step
   constexpr int RSPAN = NM / 2;        // MFMA slots over which the fragment reads of a step are spread
   const int wave = c.wave, lane = c.lane, wm = c.wm, wn = c.wn, nk = c.nk;
+  const int e = t.e, row_base = t.row_base, rows_e = t.rows_e, m0 = t.m0, n0 = t.n0;
 
-  // Ring fills address global memory through buffer resources: a scalar base per operand, a
-  // loop-invariant 32-bit byte offset per lane and fill instruction, and the k offset as scalar offset
-  // plus immediate.  Fill instruction q of a tile covers rows [16q, 16q+16); tail rows re-read the last
-  // valid row.
-  const bool gathered = p.gather_a != nullptr;
-  const uint8_t *xbase = gathered ? p.a : p.a + static_cast<int64_t>(row_base + m0) * c.kbytes;
-  const int64_t xrows = gathered ? p.a_rows : rows_e - m0;
-  const int64_t xbytes = xrows > 0 ? xrows * c.kbytes : 0xffffffffll;
-  const uint8_t *wbase = p.b + (static_cast<int64_t>(e) * p.n + n0) * c.kbytes;
-  const int64_t wbytes = static_cast<int64_t>(p.n - n0) * c.kbytes;
-  // An odd number of k-steps is rounded up by a phantom step whose fragments come from a page of zeros
-  // (every lane at offset 16 * lane).
-  const __amdgpu_buffer_rsrc_t xrsrc = make_rsrc(xbase, xbytes);
-  const __amdgpu_buffer_rsrc_t wrsrc = make_rsrc(wbase, wbytes);
+  // Operand addressing: prepared by the previous tile together with the first fills, or set up here.
+  bool prefetched = false;
+  TileOperands<XLOADS, WLOADS> op;
+  if constexpr (MB == 4 && NB == 4) {
+    if (pf.valid) {
+      prefetched = true;
+      op = pf.op;
+    }
+  }
+  if (!prefetched) setup_operands<XLOADS, WLOADS>(p, c, t, op);
+  const __amdgpu_buffer_rsrc_t xrsrc = op.xrsrc, wrsrc = op.wrsrc;
   const __amdgpu_buffer_rsrc_t zrsrc = make_rsrc(g_zero_page, 1024);
   const uint32_t zoff = lane * 16;
   uint32_t xoff[XLOADS], woff[WLOADS];
 #pragma unroll
-  for (int j = 0; j < XLOADS; ++j) {
-    int xr = m0 + (XLOADS * wave + j) * 16 + c.fill_row;
-    if (xr > rows_e - 1) xr = rows_e - 1;
-    int64_t arow = xr - m0;
-    if (gathered) {
-      arow = p.gather_a[row_base + xr];
-      if (p.a_rows > 0) arow = arow < 0 ? 0 : (arow >= p.a_rows ? p.a_rows - 1 : arow);
-    }
-    xoff[j] = static_cast<uint32_t>(arow * c.kbytes) + c.fill_chunk * 16;
-  }
+  for (int j = 0; j < XLOADS; ++j) xoff[j] = op.xoff[j];
 #pragma unroll
-  for (int j = 0; j < WLOADS; ++j) {
-    int wr = n0 + (WLOADS * wave + j) * 16 + c.fill_row;
-    if (wr > p.n - 1) wr = p.n - 1;
-    woff[j] = static_cast<uint32_t>((wr - n0) * c.kbytes) + c.fill_chunk * 16;
-  }
+  for (int j = 0; j < WLOADS; ++j) woff[j] = op.woff[j];
   // LDS destinations of this wave's fill instructions inside a stage (X rows first, then W rows).
   uint8_t *xdst = smem + (XLOADS * wave) * 1024;
   uint8_t *wdst = smem + X_TILE_BYTES + (WLOADS * wave) * 1024;
@@ -404,15 +473,9 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
     __builtin_amdgcn_sched_barrier(0);
   };
 
-  // ---- prologue: request k-steps 0..3 as two pairs, wait for the first pair ------------------------
-  FLUXMI_WAITCNT(0, 0);  // stores of the previous tile's epilogue
-  static_for<0, 2>([&](auto P) {
-    constexpr int s = 2 * decltype(P)::value;
-    static_for<0, LOADS>([&](auto Q) {
-      fill_dyn(s, Q, s);
-      fill_dyn(s + 1, Q, s + 1);
-    });
-  });
+  // ---- prologue: k-steps 0..3 requested as two pairs, here or by the previous tile ahead of its epilogue --
+  FLUXMI_WAITCNT(0, 0);  // stores of the previous tile's epilogue (and, if it requested them, the first fills)
+  if (!prefetched) issue_first_pairs<XLOADS, WLOADS>(op, smem, c);
   FLUXMI_WAITCNT(2 * LOADS, 15);
   __builtin_amdgcn_s_barrier();
   static_for<0, NR>([&](auto R) { read_one(std::integral_constant<int, 0>{}, R, xa, wa); });
@@ -445,7 +508,15 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
   // ---- epilogue ---------------------------------------------------------------------------------
   FLUXMI_WAITCNT(0, 0);          // this wave's trailing ring fills have landed
   __builtin_amdgcn_s_barrier();  // ... and everybody else's; nobody reads the ring any more
-  uint8_t *windows = smem + wave * 16384;  // two 8 KiB windows per wave
+  // A whole macro tile next: its first four k-steps are requested now, into ring slots 0..3; the
+  // epilogue's LDS windows lie in slot 4.
+  pf.valid = false;
+  if (next.kind == 0) {
+    setup_operands<4, 4>(p, c, next, pf.op);
+    issue_first_pairs<4, 4>(pf.op, smem, c);
+    pf.valid = true;
+  }
+  uint8_t *windows = smem + 4 * STAGE_BYTES + wave * 8192;  // one 8 KiB window per wave
   const int wrow0 = m0 + wm * (32 * MB);
   const int wcol0 = n0 + wn * (32 * NB);
   {
@@ -551,7 +622,10 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
   int rows_e = expert_rows(p, 0, 0);
   int tiles_e = ((rows_e + BM - 1) / BM) * tiles_n;
 
-  for (int item = virt; item < total_items; item += grid) {
+  // Work item -> tile (items must be asked for in increasing order).
+  auto locate = [&](int item) {
+    TileDesc t = {-2, 0, 0, 0, 0, 0};
+    if (item >= total_items) return t;
     int tile = item, piece = 0;
     if (item >= full_items) {
       tile = full_items + (item - full_items) / pieces;
@@ -566,7 +640,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
         tiles_e = ((rows_e + BM - 1) / BM) * tiles_n;
       }
     }
-    if (e >= p.nexperts) break;
+    if (e >= p.nexperts) return t;
     // Order inside an expert: row tiles are cut into groups of at most 8; a group is walked
     // column-major over all weight panels before the next group starts.  32 consecutive tiles (one
     // XCD's share of a round) then cover about 8 row tiles x 4 panels: 12 distinct operand tiles per
@@ -581,21 +655,37 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
     const int in_group = local - group * gm * tiles_n;
     const int nt = in_group / group_rows;
     const int mt = group_first + (in_group - nt * group_rows);
-    int m0 = mt * BM;
-    int n0 = nt * BN;
-
+    t.e = e;
+    t.row_base = row_base;
+    t.rows_e = rows_e;
+    t.m0 = mt * BM;
+    t.n0 = nt * BN;
     if (item < full_items || pieces == 1) {
       // The last row tile of an expert is run 128 rows high when that covers its rows.
-      if (rows_e - m0 > 128) gemm_tile<ELT, 4, 4>(p, smem, c, e, row_base, rows_e, m0, n0);
-      else gemm_tile<ELT, 2, 4>(p, smem, c, e, row_base, rows_e, m0, n0);
+      t.kind = rows_e - t.m0 > 128 ? 0 : 1;
     } else if (pieces == 2) {
-      n0 += piece * 128;
-      if (n0 < p.n) gemm_tile<ELT, 4, 2>(p, smem, c, e, row_base, rows_e, m0, n0);
+      t.n0 += piece * 128;
+      t.kind = t.n0 < p.n ? 2 : -1;
     } else {
-      m0 += (piece >> 1) * 128;
-      n0 += (piece & 1) * 128;
-      if (m0 < rows_e && n0 < p.n) gemm_tile<ELT, 2, 2>(p, smem, c, e, row_base, rows_e, m0, n0);
+      t.m0 += (piece >> 1) * 128;
+      t.n0 += (piece & 1) * 128;
+      t.kind = (t.m0 < rows_e && t.n0 < p.n) ? 3 : -1;
     }
+    return t;
+  };
+
+  TilePrefetch pf;
+  pf.valid = false;
+  int item = virt;
+  TileDesc cur = locate(item);
+  while (cur.kind != -2) {
+    item += grid;
+    const TileDesc next = locate(item);
+    if (cur.kind == 0) gemm_tile<ELT, 4, 4>(p, smem, c, cur, next, pf);
+    else if (cur.kind == 1) gemm_tile<ELT, 2, 4>(p, smem, c, cur, next, pf);
+    else if (cur.kind == 2) gemm_tile<ELT, 4, 2>(p, smem, c, cur, next, pf);
+    else if (cur.kind == 3) gemm_tile<ELT, 2, 2>(p, smem, c, cur, next, pf);
+    cur = next;
   }
 }
 
