@@ -19,7 +19,8 @@ EXPORTS = (
     "fluxmi_version", "fluxmi_last_error", "fluxmi_device_cu_count",
     "fluxmi_moe_route_sort_workspace_bytes", "fluxmi_moe_route_sort", "fluxmi_moe_gather_index",
     "fluxmi_grouped_gemm_workspace_bytes", "fluxmi_grouped_gemm",
-    "fluxmi_topk_gather_reduce", "fluxmi_quant_e4m3_rowwise",
+    "fluxmi_topk_gather_reduce", "fluxmi_quant_e4m3_rowwise", "fluxmi_quant_e4m3_square",
+    "fluxmi_quant_e4m3_block128",
 )
 
 
@@ -61,6 +62,8 @@ def load():
     lib.fluxmi_grouped_gemm.argtypes = [ctypes.POINTER(GroupedGemmArgs), vp, sz, vp]
     lib.fluxmi_topk_gather_reduce.argtypes = [ctypes.POINTER(vp), i32, i32, vp, vp, f32, i32, i32, i32, vp, vp]
     lib.fluxmi_quant_e4m3_rowwise.argtypes = [vp, i64, i64, i32, f32, vp, vp, i32, vp]
+    lib.fluxmi_quant_e4m3_square.argtypes = [vp, i64, i64, i64, f32, vp, vp, vp, vp, vp]
+    lib.fluxmi_quant_e4m3_block128.argtypes = [vp, i64, i64, f32, vp, vp, vp, vp, vp]
     _lib = lib
     return lib
 
@@ -202,3 +205,44 @@ def quant_e4m3(x, block_cols=0, eps=0.0, permute_scale=False):
     _check(lib.fluxmi_quant_e4m3_rowwise(_ptr(x), rows, cols, block_cols, float(eps), _ptr(q), _ptr(si),
                                          int(permute_scale), _stream()), "fluxmi_quant_e4m3_rowwise")
     return q, si
+
+
+def quant_e4m3_square(x, eps=0.0, transpose=False):
+    """x [rows, cols] or [batch, rows, cols] bf16 -> (q, scale_inv [.., rows/128, cols/128], q_t, scale_inv_t);
+    the last two are None without `transpose`.  One scale per 128 x 128 block."""
+    lib = load()
+    _dev_tensor(x, torch.bfloat16, "x")
+    lead = tuple(x.shape[:-2])
+    if len(lead) > 1:
+        raise ValueError("x must have 2 or 3 dimensions")
+    batch = lead[0] if lead else 1
+    rows, cols = x.shape[-2:]
+    nby, nbx = (rows + 127) // 128, (cols + 127) // 128
+    q = torch.empty(*lead, rows, cols, dtype=torch.float8_e4m3fn, device=x.device)
+    si = torch.empty(*lead, nby, nbx, dtype=torch.float32, device=x.device)
+    qt = sit = None
+    if transpose:
+        qt = torch.empty(*lead, cols, rows, dtype=torch.float8_e4m3fn, device=x.device)
+        sit = torch.empty(*lead, nbx, nby, dtype=torch.float32, device=x.device)
+    _check(lib.fluxmi_quant_e4m3_square(_ptr(x), batch, rows, cols, float(eps), _ptr(q), _ptr(si), _ptr(qt), _ptr(sit),
+                                        _stream()), "fluxmi_quant_e4m3_square")
+    return q, si, qt, sit
+
+
+def quant_e4m3_block128(x, eps=0.0, transpose=False):
+    """x [rows, cols] bf16 -> (q, scale_inv [rows/128, cols/128, 128], q_t [cols, rows], scale_inv_t
+    [cols/128, rows/128, 128]); the last two are None without `transpose`.  One scale per (row, 128 columns);
+    the transposed output has one per (column, 128 rows)."""
+    lib = load()
+    _dev_tensor(x, torch.bfloat16, "x")
+    rows, cols = x.shape
+    nby, nbx = (rows + 127) // 128, (cols + 127) // 128
+    q = torch.empty(rows, cols, dtype=torch.float8_e4m3fn, device=x.device)
+    si = torch.zeros(nby, nbx, 128, dtype=torch.float32, device=x.device)
+    qt = sit = None
+    if transpose:
+        qt = torch.empty(cols, rows, dtype=torch.float8_e4m3fn, device=x.device)
+        sit = torch.zeros(nbx, nby, 128, dtype=torch.float32, device=x.device)
+    _check(lib.fluxmi_quant_e4m3_block128(_ptr(x), rows, cols, float(eps), _ptr(q), _ptr(si), _ptr(qt), _ptr(sit),
+                                          _stream()), "fluxmi_quant_e4m3_block128")
+    return q, si, qt, sit

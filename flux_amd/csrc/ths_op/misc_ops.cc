@@ -31,29 +31,53 @@ Quantization::Result Quantization::quantize_vector_blockwise(torch::Tensor input
   // [ceil(M/128), ceil(K/128), 128] with the row inside its 128-row block fastest
   // (quantization.cc:91-93, quantization.cu:612-621).  Padding rows of the last block stay zero.
   torch::Tensor scale = torch::zeros({by, bx, kBlock}, input.options().dtype(at::kFloat));
-  quant_call(input, kBlock, eps, out, scale, true);
   std::optional<torch::Tensor> out_t, scale_t;
   if (return_transpose) {
-    // Column-wise scales: the same kernel on the transposed matrix.
-    torch::Tensor xt = input.t().contiguous();
-    torch::Tensor ot = torch::empty({cols, rows}, input.options().dtype(output_dtype_));
-    torch::Tensor st = torch::zeros({bx, by, kBlock}, input.options().dtype(at::kFloat));
-    quant_call(xt, kBlock, eps, ot, st, true);
-    out_t = ot;
-    scale_t = st;
+    // The transposed matrix with one scale per (column, 128-row block), from the same read of the input.
+    out_t = torch::empty({cols, rows}, input.options().dtype(output_dtype_));
+    scale_t = torch::zeros({bx, by, kBlock}, input.options().dtype(at::kFloat));
   }
+  check_status(fluxmi_quant_e4m3_block128(input.data_ptr(), rows, cols, eps, out.data_ptr(), scale.data_ptr<float>(),
+                                          return_transpose ? out_t->data_ptr() : nullptr,
+                                          return_transpose ? scale_t->data_ptr<float>() : nullptr, current_stream()),
+               "fluxmi_quant_e4m3_block128");
   return {out, scale, out_t, scale_t};
 }
 
-Quantization::Result Quantization::quantize_square_blockwise(torch::Tensor, bool, float) {
-  TORCH_CHECK(false, "quantize_square_blockwise (128x128 blocks) is not built: the MoE path uses per-row and "
-                     "1x128 scales (quantize_rowwise / quantize_vector_blockwise)");
-  return {};
+// One scale per 128 x 128 block; `input` is [batch, rows, cols] (quantization.cc:152-221 is batch = 1,
+// :228-316 loops over the batch on side streams: here the batch is one launch on the current stream).
+static Quantization::Result quant_square(const torch::Tensor &input, int64_t batch, int64_t rows, int64_t cols,
+                                         bool batched, bool return_transpose, float eps, at::ScalarType out_dtype) {
+  const int64_t bx = (cols + kBlock - 1) / kBlock, by = (rows + kBlock - 1) / kBlock;
+  auto shape = [&](int64_t a, int64_t b) {
+    return batched ? std::vector<int64_t>{batch, a, b} : std::vector<int64_t>{a, b};
+  };
+  torch::Tensor out = torch::empty(shape(rows, cols), input.options().dtype(out_dtype));
+  torch::Tensor scale = torch::empty(shape(by, bx), input.options().dtype(at::kFloat));
+  std::optional<torch::Tensor> out_t, scale_t;
+  if (return_transpose) {
+    out_t = torch::empty(shape(cols, rows), input.options().dtype(out_dtype));
+    scale_t = torch::empty(shape(bx, by), input.options().dtype(at::kFloat));
+  }
+  check_status(fluxmi_quant_e4m3_square(input.data_ptr(), batch, rows, cols, eps, out.data_ptr(),
+                                        scale.data_ptr<float>(), return_transpose ? out_t->data_ptr() : nullptr,
+                                        return_transpose ? scale_t->data_ptr<float>() : nullptr, current_stream()),
+               "fluxmi_quant_e4m3_square");
+  return {out, scale, out_t, scale_t};
 }
 
-Quantization::Result Quantization::batch_quantize_square_blockwise(torch::Tensor, bool, float) {
-  TORCH_CHECK(false, "batch_quantize_square_blockwise (128x128 blocks) is not built");
-  return {};
+Quantization::Result Quantization::quantize_square_blockwise(torch::Tensor input, bool return_transpose, float eps) {
+  TORCH_CHECK(input.dim() == 2, "Input must have 2 dimensions.");
+  FLUX_AMD_CHECK_INPUT(input, input_dtype_);
+  return quant_square(input, 1, input.size(0), input.size(1), false, return_transpose, eps, output_dtype_);
+}
+
+Quantization::Result Quantization::batch_quantize_square_blockwise(torch::Tensor input, bool return_transpose,
+                                                                   float eps) {
+  TORCH_CHECK(input.dim() == 3, "Input must have 3 dimensions.");
+  FLUX_AMD_CHECK_INPUT(input, input_dtype_);
+  return quant_square(input, input.size(0), input.size(1), input.size(2), true, return_transpose, eps,
+                      output_dtype_);
 }
 
 std::tuple<torch::Tensor, torch::Tensor> Quantization::quantize_rowwise(torch::Tensor input, float eps) {

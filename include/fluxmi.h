@@ -150,6 +150,42 @@ int fluxmi_quant_e4m3_rowwise(const void *x_bf16, int64_t rows, int64_t cols, in
                               float eps, void *q_out, float *scale_inv_out, int32_t permute_scale,
                               void *stream);
 
+/* ------------------------------------------------------------------------------------------------
+ * bf16 -> fp8-e4m3 absmax quantisation with one scale per 128 x 128 block of each [rows, cols] matrix of
+ * a batch, and optionally a transposed copy of the bytes.
+ *
+ * Stands in for `block_scaled_cast_transpose_impl` behind `Quantization::quantize_square_blockwise`
+ * (batch = 1) and `Quantization::batch_quantize_square_blockwise` (src/quantization/quantization.cu:1185-1380
+ * full blocks, :971-1183 ragged blocks, :1458-1528 dispatch; src/quantization/ths_op/quantization.cc:152-316):
+ *   amax, scale, q as for fluxmi_quant_e4m3_rowwise, taken over the part of the block inside the matrix;
+ *   scale_inv = 1.0f / scale (fp32 division).
+ * x is [batch, rows, cols] bf16; q_out [batch, rows, cols] bytes; scale_inv_out
+ * [batch, ceil(rows/128), ceil(cols/128)].  With q_t_out / scale_inv_t_out (both or neither):
+ * q_t_out[b, c, r] = q_out[b, r, c] and scale_inv_t_out [batch, ceil(cols/128), ceil(rows/128)] holds the
+ * same scales transposed.  Any rows / cols; 16-byte accesses are used when cols % 8 == 0 (and, for the
+ * transposed copy, rows % 16 == 0) and the pointers are aligned accordingly.
+ * ---------------------------------------------------------------------------------------------- */
+int fluxmi_quant_e4m3_square(const void *x_bf16, int64_t batch, int64_t rows, int64_t cols, float eps,
+                             void *q_out, float *scale_inv_out, void *q_t_out, float *scale_inv_t_out,
+                             void *stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * bf16 -> fp8-e4m3 absmax quantisation with one scale per (row, 128-column block) and, optionally, the
+ * transposed matrix quantised with one scale per (column, 128-row block), from a single read of x.
+ *
+ * Stands in for `block_scaled_1d_cast_transpose_impl` behind `Quantization::quantize_vector_blockwise`
+ * including its `return_transpose` outputs (src/quantization/quantization.cu:421-706 ragged, :708-969 full
+ * blocks, :1382-1456 dispatch; src/quantization/ths_op/quantization.cc:75-145).  Arithmetic as for
+ * fluxmi_quant_e4m3_rowwise (scale_inv = float(1.0 / double(scale))); what lies outside the matrix counts as 0.
+ *   q_out [rows, cols], scale_inv_out [ceil(rows/128), ceil(cols/128), 128] (row inside its block fastest;
+ *   entries of rows past the end are not written);
+ *   q_t_out [cols, rows], scale_inv_t_out [ceil(cols/128), ceil(rows/128), 128] (both or neither):
+ *   q_t_out[c, r] = e4m3(x[r, c] * scale_t(c, r / 128)).
+ * Any rows / cols; 16-byte accesses when cols % 8 == 0 (transposed: rows % 16 == 0) and aligned pointers.
+ * ---------------------------------------------------------------------------------------------- */
+int fluxmi_quant_e4m3_block128(const void *x_bf16, int64_t rows, int64_t cols, float eps, void *q_out,
+                               float *scale_inv_out, void *q_t_out, float *scale_inv_t_out, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

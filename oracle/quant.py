@@ -21,7 +21,8 @@ def build():
 def clib():
     global _lib
     if _lib is None:
-        if not os.path.exists(_SO):
+        src = os.path.join(_HERE, "quant_ref.c")
+        if not os.path.exists(_SO) or (os.path.exists(src) and os.path.getmtime(src) > os.path.getmtime(_SO)):
             build()
         lib = ctypes.CDLL(_SO)
         lib.fluxref_compute_scale.restype = ctypes.c_float
@@ -33,6 +34,9 @@ def clib():
         lib.fluxref_quant_rows.restype = None
         lib.fluxref_quant_rows.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int32,
                                            ctypes.c_float, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32]
+        lib.fluxref_quant_square.restype = None
+        lib.fluxref_quant_square.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_float,
+                                             ctypes.c_void_p, ctypes.c_void_p]
         _lib = lib
     return _lib
 
@@ -137,4 +141,37 @@ def quant_rows_c(x_bits, block_cols=0, eps=0.0, permute=False):
         inv = np.zeros((rows, nb), dtype=np.float32)
     lib.fluxref_quant_rows(x_bits.ctypes.data, rows, cols, block_cols, eps, q.ctypes.data, inv.ctypes.data,
                            int(permute))
+    return q, inv
+
+
+def quant_square(x_bits, eps=0.0):
+    """numpy form of the 128 x 128 block quantisation (src/quantization/quantization.cu:971-1183 ragged blocks,
+    :1185-1380 full blocks): amax over the part of a block inside the matrix, scale_inv = 1.0f / scale.
+    x_bits: uint16 bf16 bit patterns [rows, cols].  Returns (q uint8 [rows, cols], scale_inv float32
+    [ceil(rows/128), ceil(cols/128)]); the transposed outputs of the reference are q.T and scale_inv.T."""
+    x_bits = np.ascontiguousarray(x_bits, dtype=np.uint16)
+    rows, cols = x_bits.shape
+    x = bf16_bits_to_f32(x_bits)
+    nby, nbx = (rows + 127) // 128, (cols + 127) // 128
+    ax = np.abs(x)
+    ax = np.where(np.isnan(ax), np.float32(0), ax)  # fmaxf ignores NaN
+    ax = np.pad(ax, ((0, nby * 128 - rows), (0, nbx * 128 - cols)))
+    amax = ax.reshape(nby, 128, nbx, 128).max(axis=(1, 3))
+    scale = compute_scale(amax, eps)
+    with np.errstate(divide="ignore"):
+        inv = (np.float32(1.0) / scale).astype(np.float32)
+    full = np.repeat(np.repeat(scale, 128, axis=0), 128, axis=1)[:rows, :cols]
+    with np.errstate(over="ignore", invalid="ignore"):
+        q = e4m3_encode((x * full).astype(np.float32))
+    return q, inv
+
+
+def quant_square_c(x_bits, eps=0.0):
+    """Same through the C restatement."""
+    lib = clib()
+    x_bits = np.ascontiguousarray(x_bits, dtype=np.uint16)
+    rows, cols = x_bits.shape
+    q = np.zeros((rows, cols), dtype=np.uint8)
+    inv = np.zeros(((rows + 127) // 128, (cols + 127) // 128), dtype=np.float32)
+    lib.fluxref_quant_square(x_bits.ctypes.data, rows, cols, eps, q.ctypes.data, inv.ctypes.data)
     return q, inv

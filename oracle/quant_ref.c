@@ -9,6 +9,7 @@
  *   scale_inv = 1.0 / scale :612-621  (double division, stored as float; permuted [M/128][K/128][128])
  *   q = OType(float(x)*scale):674-676 (CUDA __nv_fp8_e4m3 constructor: round-nearest-even, saturate-finite)
  *   padding counts as 0     :519-525
+ *   128 x 128 blocks        :971-1183 (ragged), :1185-1380 (full); scale_inv = 1.0f / scale :1117, :1290
  */
 #include <math.h>
 #include <stdint.h>
@@ -97,6 +98,26 @@ void fluxref_quant_rows(const uint16_t *x, int64_t rows, int64_t cols, int32_t b
         float v = bf16_to_f32(x[r * cols + c]) * scale;
         q[r * cols + c] = fluxref_f32_to_e4m3(v);
       }
+    }
+  }
+}
+
+/* One scale per 128 x 128 block, taken over the part of the block inside the matrix;
+ * scale_inv[ceil(rows/128)][ceil(cols/128)]. */
+void fluxref_quant_square(const uint16_t *x, int64_t rows, int64_t cols, float eps, uint8_t *q,
+                          float *scale_inv) {
+  int64_t nby = (rows + 127) / 128, nbx = (cols + 127) / 128;
+  for (int64_t by = 0; by < nby; ++by) {
+    for (int64_t bx = 0; bx < nbx; ++bx) {
+      int64_t r1 = by * 128 + 128 < rows ? by * 128 + 128 : rows;
+      int64_t c1 = bx * 128 + 128 < cols ? bx * 128 + 128 : cols;
+      float amax = 0.f;
+      for (int64_t r = by * 128; r < r1; ++r)
+        for (int64_t c = bx * 128; c < c1; ++c) amax = max_ignore_nan(amax, fabsf(bf16_to_f32(x[r * cols + c])));
+      float scale = fluxref_compute_scale(amax, eps);
+      scale_inv[by * nbx + bx] = 1.0f / scale;
+      for (int64_t r = by * 128; r < r1; ++r)
+        for (int64_t c = bx * 128; c < c1; ++c) q[r * cols + c] = fluxref_f32_to_e4m3(bf16_to_f32(x[r * cols + c]) * scale);
     }
   }
 }

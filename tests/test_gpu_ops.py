@@ -140,6 +140,29 @@ def test_quantization_op():
     assert np.array_equal(qr.view(torch.uint8).cpu().numpy(), rq0) and np.array_equal(sr.cpu().numpy(), rs0)
 
 
+def test_quantization_square_ops():
+    """quantize_square_blockwise / batch_quantize_square_blockwise: shapes, dtypes and values of the four results."""
+    q = flux_amd.Quantization(torch.bfloat16, torch.float8_e4m3fn)
+    g = torch.Generator().manual_seed(10)
+    x = (torch.randn(3, 200, 384, generator=g) * 3).to(torch.bfloat16)
+    bits = x.view(torch.int16).numpy().view(np.uint16)
+    out, scale, out_t, scale_t = q.quantize_square_blockwise(x[0].cuda(), return_tranpose=True)
+    rq, rs = quant.quant_square_c(bits[0])
+    assert out.dtype == torch.float8_e4m3fn and tuple(out.shape) == (200, 384) and tuple(scale.shape) == (2, 3)
+    assert tuple(out_t.shape) == (384, 200) and tuple(scale_t.shape) == (3, 2)
+    assert np.array_equal(out.view(torch.uint8).cpu().numpy(), rq) and np.array_equal(scale.cpu().numpy(), rs)
+    assert np.array_equal(out_t.view(torch.uint8).cpu().numpy(), rq.T) and np.array_equal(scale_t.cpu().numpy(), rs.T)
+    out2, scale2, none_t, none_s = q.quantize_square_blockwise(x[0].cuda(), return_tranpose=False)
+    assert none_t is None and none_s is None and torch.equal(out2.view(torch.uint8), out.view(torch.uint8))
+    bo, bs, bot, bst = q.batch_quantize_square_blockwise(x.cuda())  # transposed outputs by default
+    assert tuple(bo.shape) == (3, 200, 384) and tuple(bs.shape) == (3, 2, 3)
+    assert tuple(bot.shape) == (3, 384, 200) and tuple(bst.shape) == (3, 3, 2)
+    for b in range(3):
+        rq, rs = quant.quant_square_c(bits[b])
+        assert np.array_equal(bo[b].view(torch.uint8).cpu().numpy(), rq) and np.array_equal(bs[b].cpu().numpy(), rs)
+        assert np.array_equal(bot[b].view(torch.uint8).cpu().numpy(), rq.T) and np.array_equal(bst[b].cpu().numpy(), rs.T)
+
+
 def test_fp8_layer1_through_ops():
     """fp8 activations and weights with per-row x per-output-channel scales (weight_scale [E, N], input_scale [M])."""
     wl = configs.make_workload("C5", tokens=128, hidden=512, ffn=256)

@@ -72,8 +72,12 @@ def test_dtype_and_device_checks():
         q.quantize_vector_blockwise(torch.zeros(4, dtype=torch.bfloat16))
     with pytest.raises(RuntimeError, match="device tensor"):
         q.quantize_vector_blockwise(torch.zeros(4, 8, dtype=torch.bfloat16))
-    with pytest.raises(RuntimeError, match="not built"):
+    with pytest.raises(RuntimeError, match="2 dimensions"):
+        q.quantize_square_blockwise(torch.zeros(2, 4, 8, dtype=torch.bfloat16))
+    with pytest.raises(RuntimeError, match="device tensor"):
         q.quantize_square_blockwise(torch.zeros(4, 8, dtype=torch.bfloat16))
+    with pytest.raises(RuntimeError, match="3 dimensions"):
+        q.batch_quantize_square_blockwise(torch.zeros(4, 8, dtype=torch.bfloat16))
     args = flux_amd.MoeArguments(max_ntokens=16, hidden=64, ffn_hidden=128, nexperts=4, topk=2,
                                  input_dtype=torch.bfloat16)
     assert (args.max_ntokens, args.hidden, args.ffn_hidden, args.nexperts, args.topk) == (16, 64, 128, 4, 2)

@@ -98,3 +98,48 @@ def test_quant_golden_fixture():
     assert np.array_equal(q, z["q_row"]) and np.array_equal(s, z["scale_inv_row"])
     q, s = quant.quant_rows_c(z["x_bits"], 128, 0.0, True)
     assert np.array_equal(q, z["q_blk"]) and np.array_equal(s, z["scale_inv_blk_perm"])
+
+
+def _bits(x):
+    return torch.from_numpy(np.asarray(x, dtype=np.float32)).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+
+
+@pytest.mark.parametrize("rows,cols", [(128, 128), (256, 384), (130, 200), (5, 3), (1, 129), (257, 127)])
+def test_quant_square_numpy_vs_c_vs_loops(rows, cols):
+    """128 x 128 blocks: the numpy and the C restatement agree, and both agree with a per-block loop built from
+    the already pinned scalar pieces (compute_scale, e4m3_encode)."""
+    rng = np.random.default_rng(rows * 977 + cols)
+    x = (rng.standard_normal((rows, cols)) * rng.uniform(0.01, 30, size=(rows, 1))).astype(np.float32)
+    bits = _bits(x)
+    q1, s1 = quant.quant_square(bits)
+    q2, s2 = quant.quant_square_c(bits)
+    assert np.array_equal(q1, q2) and np.array_equal(s1, s2)
+    xf = quant.bf16_bits_to_f32(bits)
+    for by in range((rows + 127) // 128):
+        for bx in range((cols + 127) // 128):
+            blk = xf[by * 128:(by + 1) * 128, bx * 128:(bx + 1) * 128]
+            scale = quant.compute_scale(np.float32(np.abs(blk).max()))
+            assert s1[by, bx] == np.float32(1.0) / scale
+            assert np.array_equal(q1[by * 128:(by + 1) * 128, bx * 128:(bx + 1) * 128],
+                                  quant.e4m3_encode((blk * scale).astype(np.float32)))
+            assert np.abs(quant.e4m3_decode(q1[by * 128:(by + 1) * 128, bx * 128:(bx + 1) * 128])).max() == 448.0
+
+
+def test_quant_square_against_row_blocks_and_special_blocks():
+    """A block's scale is the smallest of its rows' 1 x 128 scales (scale_inv: the largest); an all-zero block
+    gets scale 1 and zero codes; NaN is skipped by the amax and encoded as NaN; eps floors the amax."""
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal((256, 256)) * rng.uniform(0.01, 30, size=(256, 1))).astype(np.float32)
+    x[128:, :128] = 0
+    x[3, 200] = np.nan
+    bits = _bits(x)
+    q, s = quant.quant_square(bits)
+    qc, sc = quant.quant_square_c(bits)
+    assert np.array_equal(q, qc) and np.array_equal(s, sc)
+    _, srow = quant.quant_rows(bits, 128, 0.0, False)           # [256, 2]
+    assert np.array_equal(s, srow.reshape(2, 128, 2).max(axis=1))
+    assert s[1, 0] == 1.0 and np.all(q[128:, :128] == 0)
+    assert q[3, 200] & 0x7F == 0x7F and np.isfinite(s).all()
+    q_eps, s_eps = quant.quant_square(bits, eps=1e4)
+    assert np.all(s_eps == np.float32(1.0) / (np.float32(448.0) / np.float32(1e4)))
+    assert np.array_equal(q_eps, quant.quant_square_c(bits, eps=1e4)[0])
