@@ -238,11 +238,12 @@ def quant_e4m3_block128(x, eps=0.0, transpose=False):
     rows, cols = x.shape
     nby, nbx = (rows + 127) // 128, (cols + 127) // 128
     q = torch.empty(rows, cols, dtype=torch.float8_e4m3fn, device=x.device)
-    si = torch.zeros(nby, nbx, 128, dtype=torch.float32, device=x.device)
+    alloc = lambda n, *shape: (torch.zeros if n % 128 else torch.empty)(*shape, dtype=torch.float32, device=x.device)
+    si = alloc(rows, nby, nbx, 128)  # entries past the last row of the last block are not written
     qt = sit = None
     if transpose:
         qt = torch.empty(cols, rows, dtype=torch.float8_e4m3fn, device=x.device)
-        sit = torch.zeros(nbx, nby, 128, dtype=torch.float32, device=x.device)
+        sit = alloc(cols, nbx, nby, 128)
     _check(lib.fluxmi_quant_e4m3_block128(_ptr(x), rows, cols, float(eps), _ptr(q), _ptr(si), _ptr(qt), _ptr(sit),
                                           _stream()), "fluxmi_quant_e4m3_block128")
     return q, si, qt, sit

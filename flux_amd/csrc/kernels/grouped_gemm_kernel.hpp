@@ -223,6 +223,19 @@ struct TileDesc {
   int kind, e, row_base, rows_e, m0, n0;
 };
 
+// Ring geometry per tile shape.  Whole and half tiles: five stages of 32 KiB, fills four k-steps ahead.  The
+// 128x128 pieces of a last round need 16 KiB per stage and have short k-steps (16 MFMAs per wave), so four
+// steps of look-ahead do not cover the memory latency: they run ten stages of 16 KiB, eight steps ahead.
+// Both stage counts divide ten, the number of k-steps over which the loop is unrolled.
+template <int MB, int NB>
+struct Ring {
+  static constexpr bool deep = MB == 2 && NB == 2;
+  static constexpr int STG = deep ? 2 * STAGES : STAGES;
+  static constexpr int XB = deep ? X_TILE_BYTES / 2 : X_TILE_BYTES;  // X part of a stage
+  static constexpr int SB = deep ? STAGE_BYTES / 2 : STAGE_BYTES;    // a stage
+  static constexpr int LA = deep ? 8 : 4;                            // look-ahead in k-steps (even)
+};
+
 // Operand addressing of a tile: buffer resources and this lane's byte offsets of its fill instructions.
 template <int XL, int WL>
 struct TileOperands {
@@ -280,19 +293,19 @@ __device__ __forceinline__ void fill_any(const TileOperands<XL, WL> &op, uint8_t
   const __amdgpu_buffer_rsrc_t zrsrc = make_rsrc(g_zero_page, 1024);
   const uint32_t zoff = c.lane * 16;
   if (q < XL)
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(in ? op.xrsrc : zrsrc, (lds_ptr_t)(smem + slot * STAGE_BYTES + (XL * c.wave + q) * 1024), 16,
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(in ? op.xrsrc : zrsrc, (lds_ptr_t)(smem + slot * Ring<XL, WL>::SB + (XL * c.wave + q) * 1024), 16,
                                              static_cast<int>(in ? op.xoff[q < XL ? q : 0] : zoff), kbyte, 0, 0);
   else
     __builtin_amdgcn_raw_ptr_buffer_load_lds(in ? op.wrsrc : zrsrc,
-                                             (lds_ptr_t)(smem + slot * STAGE_BYTES + X_TILE_BYTES + (WL * c.wave + (q - XL)) * 1024), 16,
+                                             (lds_ptr_t)(smem + slot * Ring<XL, WL>::SB + Ring<XL, WL>::XB + (WL * c.wave + (q - XL)) * 1024), 16,
                                              static_cast<int>(in ? op.woff[q >= XL ? q - XL : 0] : zoff), kbyte, 0, 0);
 }
 
-// Requests k-steps 0..3 of a tile as two pairs into ring slots 0..3 (q is a constant after unrolling).
+// Requests the first LA k-steps of a tile pair by pair into ring slots 0..LA-1 (q is a constant after unrolling).
 template <int XL, int WL>
 __device__ __forceinline__ void issue_first_pairs(const TileOperands<XL, WL> &op, uint8_t *smem, const TileCtx &c) {
 #pragma unroll
-  for (int s = 0; s < 4; s += 2) {
+  for (int s = 0; s < Ring<XL, WL>::LA; s += 2) {
 #pragma unroll
     for (int q = 0; q < XL + WL; ++q) {
       fill_any<XL, WL>(op, smem, c, q, s, s);
@@ -311,6 +324,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
   constexpr int XLOADS = MB;           // direct-to-LDS instructions per wave per stage, X tile
   constexpr int WLOADS = NB;           // same, W tile
   constexpr int LOADS = XLOADS + WLOADS;
+  constexpr int STG = Ring<MB, NB>::STG, SB = Ring<MB, NB>::SB, XB = Ring<MB, NB>::XB, LA = Ring<MB, NB>::LA;
   constexpr int BLK = Geom<ELT>::BLK, NCH = Geom<ELT>::NCH;
   constexpr int MBK = 32 * MB / BLK, NBK = 32 * NB / BLK;  // operand blocks of a wave
   constexpr int NR = (MBK + NBK) * NCH;  // fragment reads per k-step (16 bytes per lane each)
@@ -339,7 +353,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
   for (int j = 0; j < WLOADS; ++j) woff[j] = op.woff[j];
   // LDS destinations of this wave's fill instructions inside a stage (X rows first, then W rows).
   uint8_t *xdst = smem + (XLOADS * wave) * 1024;
-  uint8_t *wdst = smem + X_TILE_BYTES + (WLOADS * wave) * 1024;
+  uint8_t *wdst = smem + XB + (WLOADS * wave) * 1024;
 
   // Fill instruction Q of the k-step at byte offset kbyte of every row, into ring slot SLOT (compile-time
   // slot: the LDS address is an immediate).  The k offset travels as the scalar offset: an instruction
@@ -347,10 +361,10 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
   auto fill_one = [&](auto SLOT, auto Q, int kbyte) {
     constexpr int slot = decltype(SLOT)::value, q = decltype(Q)::value;
     if constexpr (q < XLOADS)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(xrsrc, (lds_ptr_t)(xdst + slot * STAGE_BYTES + q * 1024), 16,
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(xrsrc, (lds_ptr_t)(xdst + slot * SB + q * 1024), 16,
                                                static_cast<int>(xoff[q]), kbyte, 0, 0);
     else
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(wrsrc, (lds_ptr_t)(wdst + slot * STAGE_BYTES + (q - XLOADS) * 1024), 16,
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(wrsrc, (lds_ptr_t)(wdst + slot * SB + (q - XLOADS) * 1024), 16,
                                                static_cast<int>(woff[q - XLOADS]), kbyte, 0, 0);
   };
   // Same with a run-time slot, for the last steps of a tile; a k-step past the end of K (the phantom
@@ -360,10 +374,10 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
     const bool in = kstep < nk;
     const int kbyte = in ? kstep * KBYTES : 0;
     if constexpr (q < XLOADS)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(in ? xrsrc : zrsrc, (lds_ptr_t)(xdst + slot * STAGE_BYTES + q * 1024), 16,
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(in ? xrsrc : zrsrc, (lds_ptr_t)(xdst + slot * SB + q * 1024), 16,
                                                static_cast<int>(in ? xoff[q] : zoff), kbyte, 0, 0);
     else
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(in ? wrsrc : zrsrc, (lds_ptr_t)(wdst + slot * STAGE_BYTES + (q - XLOADS) * 1024),
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(in ? wrsrc : zrsrc, (lds_ptr_t)(wdst + slot * SB + (q - XLOADS) * 1024),
                                                16, static_cast<int>(in ? woff[q - XLOADS] : zoff), kbyte, 0, 0);
   };
 
@@ -383,7 +397,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
 #pragma unroll
     for (int s = 0; s < NCH; ++s) {
       xfrag[hi][s] = smem + hi * 65536 + wm * (32 * MB) * KBYTES + c.frag_off[s];
-      wfrag[hi][s] = smem + hi * 65536 + X_TILE_BYTES + wn * (32 * NB) * KBYTES + c.frag_off[s];
+      wfrag[hi][s] = smem + hi * 65536 + XB + wn * (32 * NB) * KBYTES + c.frag_off[s];
     }
   i32x4 xa[MBK][NCH], wa[NBK][NCH], xb[MBK][NCH], wb[NBK][NCH];
   // Fragment read R of the k-step in ring slot SLOT: chunk s = R / (MBK + NBK) of W block q (q < NBK) or of
@@ -391,7 +405,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
   auto read_one = [&](auto SLOT, auto R, i32x4 (&xf)[MBK][NCH], i32x4 (&wf)[NBK][NCH]) {
     constexpr int slot = decltype(SLOT)::value, r = decltype(R)::value;
     constexpr int s = r / (MBK + NBK), q = r % (MBK + NBK);
-    constexpr int hi = (slot * STAGE_BYTES) / 65536, lo = (slot * STAGE_BYTES) % 65536;
+    constexpr int hi = (slot * SB) / 65536, lo = (slot * SB) % 65536;
     if constexpr (q < NBK) wf[q][s] = *reinterpret_cast<const i32x4 *>(wfrag[hi][s] + lo + q * BLK * KBYTES);
     else xf[q - NBK][s] = *reinterpret_cast<const i32x4 *>(xfrag[hi][s] + lo + (q - NBK) * BLK * KBYTES);
   };
@@ -399,8 +413,8 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
   auto read_dyn = [&](int slot, auto R, i32x4 (&xf)[MBK][NCH], i32x4 (&wf)[NBK][NCH]) {
     constexpr int r = decltype(R)::value;
     constexpr int s = r / (MBK + NBK), q = r % (MBK + NBK);
-    if constexpr (q < NBK) wf[q][s] = *reinterpret_cast<const i32x4 *>(wfrag[0][s] + slot * STAGE_BYTES + q * BLK * KBYTES);
-    else xf[q - NBK][s] = *reinterpret_cast<const i32x4 *>(xfrag[0][s] + slot * STAGE_BYTES + (q - NBK) * BLK * KBYTES);
+    if constexpr (q < NBK) wf[q][s] = *reinterpret_cast<const i32x4 *>(wfrag[0][s] + slot * SB + q * BLK * KBYTES);
+    else xf[q - NBK][s] = *reinterpret_cast<const i32x4 *>(xfrag[0][s] + slot * SB + (q - NBK) * BLK * KBYTES);
   };
 
   // One k-step, number U within a run of ten (ring of five slots x two fragment sets: after ten steps
@@ -415,9 +429,9 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
     constexpr int e0 = u & ~1;
     // Stage u+1 has landed once the pair it belongs to is complete; fills are counted in issue order.
     if constexpr (even) {
-      FLUXMI_WAITCNT(2 * LOADS, 15);  // all but the pair requested during the last two steps
+      FLUXMI_WAITCNT((LA - 2) * LOADS, 15);  // all but the pairs requested since the one stage u+1 is in
     } else {
-      FLUXMI_WAITCNT(LOADS, 15);      // all but the half pair requested during the last step
+      FLUXMI_WAITCNT((LA - 3) * LOADS, 15);  // ... and the half pair requested during the last step
     }
     __builtin_amdgcn_s_barrier();     // ... for every wave's share; and everybody is done reading stage u
     __builtin_amdgcn_sched_barrier(0);
@@ -425,13 +439,13 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
       constexpr int t = decltype(T)::value;
       static_for<0, NR>([&](auto R) {
         constexpr int r = decltype(R)::value;
-        if constexpr (r * RSPAN / NR == t) read_one(std::integral_constant<int, (u + 1) % STAGES>{}, R, xn, wn_);
+        if constexpr (r * RSPAN / NR == t) read_one(std::integral_constant<int, (u + 1) % STG>{}, R, xn, wn_);
       });
       static_for<0, 2 * LOADS>([&](auto D) {
         constexpr int d = decltype(D)::value;
         if constexpr ((d * (2 * NM) / (2 * LOADS) + 1) % (2 * NM) == t + (even ? 0 : NM))
-          fill_one(std::integral_constant<int, (e0 + 4 + (d & 1)) % STAGES>{}, std::integral_constant<int, (d >> 1)>{},
-                   kbase + (e0 + 4 + (d & 1)) * KBYTES);
+          fill_one(std::integral_constant<int, (e0 + LA + (d & 1)) % STG>{}, std::integral_constant<int, (d >> 1)>{},
+                   kbase + (e0 + LA + (d & 1)) * KBYTES);
       });
       mfma_slot<ELT, MBK, NBK>(t, xc, wc, acc);
       __builtin_amdgcn_sched_barrier(0);
@@ -443,14 +457,14 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
   // number is not a multiple of ten.
   auto step_dyn = [&](int ks, bool even, i32x4 (&xc)[MBK][NCH], i32x4 (&wc)[NBK][NCH], i32x4 (&xn)[MBK][NCH], i32x4 (&wn_)[NBK][NCH]) {
     if (even) {
-      FLUXMI_WAITCNT(2 * LOADS, 15);
+      FLUXMI_WAITCNT((LA - 2) * LOADS, 15);
     } else {
-      FLUXMI_WAITCNT(LOADS, 15);
+      FLUXMI_WAITCNT((LA - 3) * LOADS, 15);
     }
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
     const int e0 = even ? ks : ks - 1;
-    const int rslot = (ks + 1) % STAGES, pslot0 = (e0 + 4) % STAGES, pslot1 = (e0 + 5) % STAGES;
+    const int rslot = (ks + 1) % STG, pslot0 = (e0 + LA) % STG, pslot1 = (e0 + LA + 1) % STG;
     static_for<0, NM>([&](auto T) {
       constexpr int t = decltype(T)::value;
       static_for<0, NR>([&](auto R) {
@@ -461,9 +475,9 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
         constexpr int d = decltype(D)::value;
         constexpr int at = (d * (2 * NM) / (2 * LOADS) + 1) % (2 * NM);
         if constexpr (at < NM) {
-          if (at == t && even) fill_dyn((d & 1) ? pslot1 : pslot0, std::integral_constant<int, (d >> 1)>{}, e0 + 4 + (d & 1));
+          if (at == t && even) fill_dyn((d & 1) ? pslot1 : pslot0, std::integral_constant<int, (d >> 1)>{}, e0 + LA + (d & 1));
         } else {
-          if (at - NM == t && !even) fill_dyn((d & 1) ? pslot1 : pslot0, std::integral_constant<int, (d >> 1)>{}, e0 + 4 + (d & 1));
+          if (at - NM == t && !even) fill_dyn((d & 1) ? pslot1 : pslot0, std::integral_constant<int, (d >> 1)>{}, e0 + LA + (d & 1));
         }
       });
       mfma_slot<ELT, MBK, NBK>(t, xc, wc, acc);
@@ -476,16 +490,16 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
   // ---- prologue: k-steps 0..3 requested as two pairs, here or by the previous tile ahead of its epilogue --
   FLUXMI_WAITCNT(0, 0);  // stores of the previous tile's epilogue (and, if it requested them, the first fills)
   if (!prefetched) issue_first_pairs<XLOADS, WLOADS>(op, smem, c);
-  FLUXMI_WAITCNT(2 * LOADS, 15);
+  FLUXMI_WAITCNT((LA - 2) * LOADS, 15);
   __builtin_amdgcn_s_barrier();
   static_for<0, NR>([&](auto R) { read_one(std::integral_constant<int, 0>{}, R, xa, wa); });
   FLUXMI_WAITCNT(63, 0);  // in registers before the first step's barrier lets anyone refill that slot
 
   // ---- main loop ----------------------------------------------------------------------------------
-  // Whole trips of ten k-steps while every k-step a trip requests (up to 13 past its first one) exists,
-  // then the remaining 4 to 23 steps pair by pair with run-time ring slots.  An odd number of k-steps
+  // Whole trips of ten k-steps while every k-step a trip requests (up to 9 + LA past its first one) exists,
+  // then the remaining steps pair by pair with run-time ring slots.  An odd number of k-steps
   // ends with a phantom step on zero fragments.
-  const int nfast = nk >= 14 ? (nk - 14) / 10 + 1 : 0;  // trips with 10 * trip + 13 < nk
+  const int nfast = nk >= 10 + LA ? (nk - (10 + LA)) / 10 + 1 : 0;  // trips with 10 * trip + 9 + LA < nk
   int kbase = 0;  // byte offset along K of step 0 of the current trip
   for (int trip = 0; trip < nfast; ++trip) {
     step(std::integral_constant<int, 0>{}, kbase, xa, wa, xb, wb);

@@ -30,12 +30,14 @@ Quantization::Result Quantization::quantize_vector_blockwise(torch::Tensor input
   torch::Tensor out = torch::empty({rows, cols}, input.options().dtype(output_dtype_));
   // [ceil(M/128), ceil(K/128), 128] with the row inside its 128-row block fastest
   // (quantization.cc:91-93, quantization.cu:612-621).  Padding rows of the last block stay zero.
-  torch::Tensor scale = torch::zeros({by, bx, kBlock}, input.options().dtype(at::kFloat));
+  // Entries of rows (columns) past the end of the last block are not written: zero-fill only when there are any.
+  auto fopt = input.options().dtype(at::kFloat);
+  torch::Tensor scale = rows % kBlock ? torch::zeros({by, bx, kBlock}, fopt) : torch::empty({by, bx, kBlock}, fopt);
   std::optional<torch::Tensor> out_t, scale_t;
   if (return_transpose) {
     // The transposed matrix with one scale per (column, 128-row block), from the same read of the input.
     out_t = torch::empty({cols, rows}, input.options().dtype(output_dtype_));
-    scale_t = torch::zeros({bx, by, kBlock}, input.options().dtype(at::kFloat));
+    scale_t = cols % kBlock ? torch::zeros({bx, by, kBlock}, fopt) : torch::empty({bx, by, kBlock}, fopt);
   }
   check_status(fluxmi_quant_e4m3_block128(input.data_ptr(), rows, cols, eps, out.data_ptr(), scale.data_ptr<float>(),
                                           return_transpose ? out_t->data_ptr() : nullptr,

@@ -106,11 +106,11 @@ def test_single_expert_matches_dense_gemm():
     assert_close(out, ref, "dense")
 
 
-@pytest.mark.parametrize("k", [96, 160, 416, 448, 480, 736, 768, 800, 1312])
+@pytest.mark.parametrize("k", [96, 160, 416, 448, 480, 544, 576, 608, 736, 768, 800, 864, 896, 928, 1312])
 def test_bf16_k_loop_boundaries(k):
     """K lengths around the seams of the k loop: odd numbers of 64-byte k-steps (a phantom step on zeros), the
-    hand-over from the unrolled trips of ten to the pair-wise tail (14 and 24 k-steps) and lengths on either
-    side; rows chosen so that full tiles, a 128-row tile and last-round pieces all occur."""
+    hand-over from the unrolled trips of ten to the pair-wise tail (14 and 24 k-steps; 18 and 28 for the
+    128x128 pieces with their deeper ring) and lengths on either side; rows chosen so that full tiles, a 128-row tile and last-round pieces all occur."""
     from flux_amd import capi
     print(f"[case] grouped_gemm bf16 k-loop seams K={k}", flush=True)
     g = torch.Generator().manual_seed(k)
