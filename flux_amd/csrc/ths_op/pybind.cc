@@ -109,4 +109,25 @@ PYBIND11_MODULE(flux_ths_pybind, m) {
         py::arg("topk"), py::arg("row_weight") = py::none(), py::arg("scale") = 1.0);
   m.def("bitwise_check", &bitwise_check);
   m.def("init_flux_shm", [](py::object) {}, py::arg("group") = py::none());  // nothing to set up on one GPU
+  // Test helper of the reference (src/ths_op/helper_ops.cc:33-44, src/cuda/random_initialize.cu:27-51): fills a
+  // half / bf16 / fp8 device tensor with uniform values of [min, max] from `seed`.  The values come from torch's
+  // generator, not from cuRAND's: the same seed gives the same tensor here, not the reference's tensor.
+  m.def("uniform_initialize", [](torch::Tensor tensor, uint64_t seed, double min, double max) {
+    const at::ScalarType st = tensor.scalar_type();
+    TORCH_CHECK(st == at::kHalf || st == at::kBFloat16 || st == at::ScalarType::Float8_e4m3fn ||
+                    st == at::ScalarType::Float8_e5m2,
+                "unsupported dtype: ", st);
+    TORCH_CHECK(tensor.is_cuda(), "uniform_initialize: tensor must be a device tensor");
+    py::object torch_mod = py::module_::import("torch");
+    py::object gen = torch_mod.attr("Generator")(py::arg("device") = tensor.device().str());
+    gen.attr("manual_seed")(seed);
+    py::object tmp = torch_mod.attr("empty")(tensor.sizes().vec(), py::arg("dtype") = torch_mod.attr("float32"),
+                                            py::arg("device") = tensor.device().str());
+    tmp.attr("uniform_")(min, max, py::arg("generator") = gen);
+    tensor.copy_(tmp.cast<torch::Tensor>());
+    return true;
+  });
+  // The reference's tuning records select among its generated kernel variants (src/ths_op/ths_op.cc:213-216);
+  // this build has one kernel per element type, so there is nothing to register.
+  m.def("load_tuning_record", [](py::object) {}, py::arg("record"));
 }

@@ -140,6 +140,19 @@ def test_quantization_op():
     assert np.array_equal(qr.view(torch.uint8).cpu().numpy(), rq0) and np.array_equal(sr.cpu().numpy(), rs0)
 
 
+def test_uniform_initialize():
+    for dt in (torch.bfloat16, torch.float16, torch.float8_e4m3fn):
+        t = torch.zeros(4096, dtype=dt, device="cuda")
+        assert flux_amd.uniform_initialize(t, 7, -0.5, 1.5)
+        f = t.float()
+        assert float(f.min()) >= -0.5 and float(f.max()) <= 1.5 and 0.3 < float(f.mean()) < 0.7
+        u = torch.zeros(4096, dtype=dt, device="cuda")
+        flux_amd.uniform_initialize(u, 7, -0.5, 1.5)
+        assert torch.equal(t.view(torch.uint8), u.view(torch.uint8))
+        flux_amd.uniform_initialize(u, 8, -0.5, 1.5)
+        assert not torch.equal(t.view(torch.uint8), u.view(torch.uint8))
+
+
 def test_quantization_square_ops():
     """quantize_square_blockwise / batch_quantize_square_blockwise: shapes, dtypes and values of the four results."""
     q = flux_amd.Quantization(torch.bfloat16, torch.float8_e4m3fn)

@@ -11,7 +11,8 @@ import flux_amd
 def test_module_exports_reference_names():
     m = flux_amd.flux_ths_pybind
     for name in ("MoeArguments", "DistEnvTPWithEP", "GemmGroupedV3AGScatter", "GemmGroupedV3GatherRS", "GemmGroupedV3",
-                 "Quantization", "calc_scatter_index", "topk_scatter_reduce", "bitwise_check", "init_flux_shm"):
+                 "Quantization", "calc_scatter_index", "topk_scatter_reduce", "bitwise_check", "init_flux_shm",
+                 "uniform_initialize", "load_tuning_record"):
         assert hasattr(m, name), name
         assert getattr(flux_amd, name) is getattr(m, name)
     for cls, methods in ((m.GemmGroupedV3AGScatter, ("forward", "forward_multiple_weights", "clear_buffers")),
@@ -60,6 +61,9 @@ def test_world_size_above_one_is_rejected():
     with pytest.raises(RuntimeError, match="nnodes"):
         flux_amd.DistEnvTPWithEP(None, 2)
     flux_amd.init_flux_shm(None)
+    flux_amd.load_tuning_record(object())
+    with pytest.raises(RuntimeError, match="unsupported dtype"):
+        flux_amd.uniform_initialize(torch.zeros(4), 1, 0.0, 1.0)
 
 
 def test_dtype_and_device_checks():
