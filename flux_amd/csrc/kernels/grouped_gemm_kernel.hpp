@@ -216,7 +216,6 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const uint8_t *base,
   const uint32_t n = bytes > 0xffffffffll ? 0xffffffffu : static_cast<uint32_t>(bytes < 0 ? 0 : bytes);
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(base), 0, static_cast<int>(n), 0x00020000);
 }
-
 // Where a work item lies.  kind: 0 a whole macro tile (4, 4); 1 the 128-row tile ending an expert (2, 4);
 // 2 a 256x128 piece (4, 2); 3 a 128x128 piece (2, 2); -1 an item without work; -2 past the last item.
 struct TileDesc {
@@ -367,6 +366,29 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
       __builtin_amdgcn_raw_ptr_buffer_load_lds(wrsrc, (lds_ptr_t)(wdst + slot * SB + (q - XLOADS) * 1024), 16,
                                                static_cast<int>(woff[q - XLOADS]), kbyte, 0, 0);
   };
+  // The same fill as two instructions placed by hand: the LDS destination goes into M0 one MFMA slot ahead
+  // of the load.  The builtin emits s_mov m0 / s_nop / buffer_load as one cluster; every instruction between
+  // two MFMAs costs about two cycles of the MFMA pipe, and set apart the pair needs no s_nop (+0.7 % end to
+  // end).  Nothing else in the k loop uses M0.
+  const uint32_t xdst32 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)xdst));
+  const uint32_t wdst32 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)wdst));
+  auto fill_m0 = [&](auto SLOT, auto Q) {
+    constexpr int slot = decltype(SLOT)::value, q = decltype(Q)::value;
+    const uint32_t dst = q < XLOADS ? xdst32 + slot * SB + q * 1024 : wdst32 + slot * SB + (q - XLOADS) * 1024;
+    asm volatile("s_mov_b32 m0, %0" : : "s"(dst) : "memory");
+  };
+  auto fill_go = [&](auto Q, int kbyte) {
+    constexpr int q = decltype(Q)::value;
+    if constexpr (q < XLOADS) {
+      const uint32_t vo = xoff[q];
+      __amdgpu_buffer_rsrc_t r = xrsrc;
+      asm volatile("buffer_load_dwordx4 %0, %1, %2 offen lds" : : "v"(vo), "s"(r), "s"(kbyte) : "memory");
+    } else {
+      const uint32_t vo = woff[q - XLOADS];
+      __amdgpu_buffer_rsrc_t r = wrsrc;
+      asm volatile("buffer_load_dwordx4 %0, %1, %2 offen lds" : : "v"(vo), "s"(r), "s"(kbyte) : "memory");
+    }
+  };
   // Same with a run-time slot, for the last steps of a tile; a k-step past the end of K (the phantom
   // second half of the last pair of an odd K) is filled from the zero page.
   auto fill_dyn = [&](int slot, auto Q, int kstep) {
@@ -443,9 +465,16 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
       });
       static_for<0, 2 * LOADS>([&](auto D) {
         constexpr int d = decltype(D)::value;
-        if constexpr ((d * (2 * NM) / (2 * LOADS) + 1) % (2 * NM) == t + (even ? 0 : NM))
+        constexpr int at = (d * (2 * NM) / (2 * LOADS) + 1) % (2 * NM);
+        if constexpr (at % NM != 0) {  // the slot before is in the same step
+          if constexpr (at - 1 == t + (even ? 0 : NM))
+            fill_m0(std::integral_constant<int, (e0 + LA + (d & 1)) % STG>{}, std::integral_constant<int, (d >> 1)>{});
+          if constexpr (at == t + (even ? 0 : NM))
+            fill_go(std::integral_constant<int, (d >> 1)>{}, kbase + (e0 + LA + (d & 1)) * KBYTES);
+        } else if constexpr (at == t + (even ? 0 : NM)) {
           fill_one(std::integral_constant<int, (e0 + LA + (d & 1)) % STG>{}, std::integral_constant<int, (d >> 1)>{},
                    kbase + (e0 + LA + (d & 1)) * KBYTES);
+        }
       });
       mfma_slot<ELT, MBK, NBK>(t, xc, wc, acc);
       __builtin_amdgcn_sched_barrier(0);
