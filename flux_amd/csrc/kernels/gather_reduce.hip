@@ -70,6 +70,10 @@ __device__ __forceinline__ void accumulate8(float (&acc)[8], const Vec8<false> &
   }
 }
 
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+  return static_cast<uint32_t>(float_to_bf16_bits(lo)) | (static_cast<uint32_t>(float_to_bf16_bits(hi)) << 16);
+}
+
 // TOPK > 0: compile-time top-k (loads fully unrolled).  TOPK == 0: run-time top-k.
 // NT: non-temporal source loads.  The choice is made once per launch and hoisted out of the load
 // sequence, so that no control flow sits between the loads of one output vector.
@@ -81,6 +85,58 @@ __device__ __forceinline__ void topk_gather_reduce_body(
   const int topk = TOPK > 0 ? TOPK : topk_rt;
   const size_t row_vecs = static_cast<size_t>(nvec);
   const int nthreads = blockDim.x;
+  if constexpr (IN_F32 && TOPK > 0) {
+    // fp32 rows: a lane takes the 16-byte units q and q + nthreads of a pass (not two adjacent ones), so that
+    // every load instruction of a wave covers 1 KiB of contiguous row, as in the bf16 case.
+    const int nq = 2 * nvec;  // 16-byte units (4 elements) per source row
+    for (int q0 = blockIdx.y * 2 * nthreads; q0 < nq; q0 += gridDim.y * 2 * nthreads) {
+      const int qa = q0 + threadIdx.x, qb = qa + nthreads;
+      const bool oka = qa < nq, okb = qb < nq;
+      u32x4 va[NGROUPS][TOPK], vb[NGROUPS][TOPK];
+      float w[TOPK];
+#pragma unroll
+      for (int j = 0; j < TOPK; ++j) {
+        const int32_t r = routing_idx[static_cast<size_t>(t) * TOPK + j];
+        w[j] = 0.f;
+        if (r >= 0) w[j] = WEIGHTED ? row_weight[r] : 1.f;
+#pragma unroll
+        for (int g = 0; g < NGROUPS; ++g) {
+          va[g][j] = u32x4{0u, 0u, 0u, 0u};
+          vb[g][j] = u32x4{0u, 0u, 0u, 0u};
+          const u32x4 *src = reinterpret_cast<const u32x4 *>(in.p[g]) + static_cast<size_t>(r < 0 ? 0 : r) * nq;
+          if (r >= 0 && oka) va[g][j] = load16<NT>(src + qa);
+          if (r >= 0 && okb) vb[g][j] = load16<NT>(src + qb);
+        }
+      }
+      float a[4] = {0.f, 0.f, 0.f, 0.f}, b[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int g = 0; g < NGROUPS; ++g) {
+#pragma unroll
+        for (int j = 0; j < TOPK; ++j) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            a[i] = fmaf(w[j], __uint_as_float(va[g][j][i]), a[i]);
+            b[i] = fmaf(w[j], __uint_as_float(vb[g][j][i]), b[i]);
+          }
+        }
+      }
+      typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+      u32x2 *dst = reinterpret_cast<u32x2 *>(out) + static_cast<size_t>(t) * nq;
+      if (oka) {
+        u32x2 o;
+        o[0] = pack2(a[0] * scale, a[1] * scale);
+        o[1] = pack2(a[2] * scale, a[3] * scale);
+        __builtin_nontemporal_store(o, dst + qa);
+      }
+      if (okb) {
+        u32x2 o;
+        o[0] = pack2(b[0] * scale, b[1] * scale);
+        o[1] = pack2(b[2] * scale, b[3] * scale);
+        __builtin_nontemporal_store(o, dst + qb);
+      }
+    }
+    return;
+  }
   for (int v = blockIdx.y * nthreads + threadIdx.x; v < nvec; v += gridDim.y * nthreads) {
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     if constexpr (TOPK > 0) {
