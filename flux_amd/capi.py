@@ -188,13 +188,26 @@ def topk_gather_reduce(inputs, routing_idx, topk, row_weight=None, scale=1.0, ou
     return out
 
 
-def quant_e4m3(x, block_cols=0, eps=0.0, permute_scale=False):
-    """-> (q fp8_e4m3fn like x, scale_inv fp32).  block_cols 0 = one scale per row, 128 = 1x128 blocks."""
+def quant_e4m3(x, block_cols=0, eps=0.0, permute_scale=False, out=None):
+    """-> (q fp8_e4m3fn like x, scale_inv fp32).  block_cols 0 = one scale per row, 128 = 1x128 blocks.
+    `out` = (q, scale_inv) of a previous call with the same arguments writes into those tensors."""
     lib = load()
     _dev_tensor(x, torch.bfloat16, "x")
     rows, cols = x.shape
-    q = torch.empty(rows, cols, dtype=torch.float8_e4m3fn, device=x.device)
-    if block_cols == 0:
+    if out is not None:
+        q, si = out
+        if q.shape != x.shape or q.dtype != torch.float8_e4m3fn or si.dtype != torch.float32 or not (
+                q.is_cuda and si.is_cuda and q.is_contiguous() and si.is_contiguous()):
+            raise ValueError("out must be the (q, scale_inv) pair of a call with the same arguments")
+        want = rows if block_cols == 0 else (
+            (rows + 127) // 128 * 128 if permute_scale else rows) * ((cols + block_cols - 1) // block_cols)
+        if si.numel() != want:
+            raise ValueError(f"scale_inv has {si.numel()} entries, expected {want}")
+    else:
+        q = torch.empty(rows, cols, dtype=torch.float8_e4m3fn, device=x.device)
+    if out is not None:
+        pass
+    elif block_cols == 0:
         si = torch.empty(rows, dtype=torch.float32, device=x.device)
     else:
         nb = (cols + block_cols - 1) // block_cols
