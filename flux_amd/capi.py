@@ -18,7 +18,7 @@ FP8_E4M3 = 1
 EXPORTS = (
     "fluxmi_version", "fluxmi_last_error", "fluxmi_device_cu_count",
     "fluxmi_moe_route_sort_workspace_bytes", "fluxmi_moe_route_sort", "fluxmi_moe_gather_index",
-    "fluxmi_grouped_gemm_workspace_bytes", "fluxmi_grouped_gemm",
+    "fluxmi_grouped_gemm_workspace_bytes", "fluxmi_grouped_gemm", "fluxmi_grouped_gemm_multi",
     "fluxmi_topk_gather_reduce", "fluxmi_quant_e4m3_rowwise", "fluxmi_quant_e4m3_square",
     "fluxmi_quant_e4m3_block128",
 )
@@ -60,6 +60,7 @@ def load():
     lib.fluxmi_grouped_gemm_workspace_bytes.restype = sz
     lib.fluxmi_grouped_gemm_workspace_bytes.argtypes = [ctypes.POINTER(GroupedGemmArgs)]
     lib.fluxmi_grouped_gemm.argtypes = [ctypes.POINTER(GroupedGemmArgs), vp, sz, vp]
+    lib.fluxmi_grouped_gemm_multi.argtypes = [ctypes.POINTER(GroupedGemmArgs), i32, vp, vp, vp, vp, sz, vp]
     lib.fluxmi_topk_gather_reduce.argtypes = [ctypes.POINTER(vp), i32, i32, vp, vp, f32, i32, i32, i32, vp, vp]
     lib.fluxmi_quant_e4m3_rowwise.argtypes = [vp, i64, i64, i32, f32, vp, vp, i32, vp]
     lib.fluxmi_quant_e4m3_square.argtypes = [vp, i64, i64, i64, f32, vp, vp, vp, vp, vp]
@@ -161,6 +162,54 @@ def grouped_gemm(a, b, splits, out=None, gather_a=None, scatter_d=None, alpha=No
         scalar_scale_dev=None if scalar_scale_dev is None else scalar_scale_dev.data_ptr())
     _check(lib.fluxmi_grouped_gemm(ctypes.byref(args), None, 0, _stream()), "fluxmi_grouped_gemm")
     return out
+
+
+def grouped_gemm_multi(a, bs, splits, outs=None, gather_a=None, alphas=None, row_scale=None, col_scale=None,
+                       scalar_scale=1.0, max_rows=None, out_dtype=None):
+    """[A @ B_g for B_g in bs] in one launch (fluxmi_grouped_gemm_multi): the same sorted rows times up to four
+    weight tensors [E, N, K], each with its own output and optional per-expert alpha."""
+    lib = load()
+    dtype = {torch.bfloat16: BF16, torch.float8_e4m3fn: FP8_E4M3}.get(a.dtype)
+    if dtype is None:
+        raise ValueError(f"unsupported input dtype {a.dtype}")
+    ng = len(bs)
+    _dev_tensor(a, a.dtype, "a")
+    for b in bs:
+        _dev_tensor(b, a.dtype, "b")
+        if b.shape != bs[0].shape:
+            raise ValueError("all weight groups must have one shape")
+    _dev_tensor(splits, torch.int32, "splits")
+    _dev_tensor(gather_a, torch.int32, "gather_a")
+    _dev_tensor(row_scale, torch.float32, "row_scale")
+    _dev_tensor(col_scale, torch.float32, "col_scale")
+    e, n, k = bs[0].shape
+    if a.shape[1] != k:
+        raise ValueError(f"K mismatch: a {tuple(a.shape)} vs b {tuple(bs[0].shape)}")
+    if max_rows is None:
+        max_rows = gather_a.numel() if gather_a is not None else a.shape[0]
+    if outs is None:
+        outs = [torch.empty(max_rows, n, dtype=out_dtype or torch.bfloat16, device=a.device) for _ in range(ng)]
+    for o in outs:
+        _dev_tensor(o, outs[0].dtype, "out")
+        if o.dtype not in (torch.bfloat16, torch.float32) or o.shape[0] < max_rows or o.shape[1] != n:
+            raise ValueError(f"out {tuple(o.shape)} {o.dtype} does not fit [{max_rows}, {n}] bf16/fp32")
+    if len(outs) != ng or (alphas is not None and len(alphas) != ng):
+        raise ValueError("outs / alphas need one entry per weight group")
+    for al in alphas or ():
+        _dev_tensor(al, torch.float32, "alpha")
+    args = GroupedGemmArgs(
+        dtype=dtype, nexperts=e, max_rows=max_rows, n=n, k=k, a_rows=a.shape[0], a=a.data_ptr(), b=None, d=None,
+        splits=splits.data_ptr(), gather_a=None if gather_a is None else gather_a.data_ptr(), scatter_d=None,
+        alpha=None, row_scale=None if row_scale is None else row_scale.data_ptr(),
+        col_scale=None if col_scale is None else col_scale.data_ptr(), scalar_scale=float(scalar_scale),
+        d_fp32=int(outs[0].dtype == torch.float32), scalar_scale_dev=None)
+    vps = ctypes.c_void_p * ng
+    b_arr = vps(*[b.data_ptr() for b in bs])
+    d_arr = vps(*[o.data_ptr() for o in outs])
+    al_arr = None if alphas is None else vps(*[None if al is None else al.data_ptr() for al in alphas])
+    _check(lib.fluxmi_grouped_gemm_multi(ctypes.byref(args), ng, b_arr, d_arr, al_arr, None, 0, _stream()),
+           "fluxmi_grouped_gemm_multi")
+    return outs
 
 
 def topk_gather_reduce(inputs, routing_idx, topk, row_weight=None, scale=1.0, out=None):

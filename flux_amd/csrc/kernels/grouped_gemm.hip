@@ -17,7 +17,7 @@ __device__ __forceinline__ float e4m3_to_float(uint8_t b) {
 }
 
 template <int ELT>
-__global__ __launch_bounds__(256) void grouped_gemm_generic_kernel(const GemmParams p) {
+__global__ __launch_bounds__(256) void grouped_gemm_generic_kernel(const GemmParams p, const int g) {
   __shared__ int32_t s_row_off[kMaxExperts + 1];
   if (threadIdx.x == 0) {
     int acc = 0;
@@ -46,7 +46,7 @@ __global__ __launch_bounds__(256) void grouped_gemm_generic_kernel(const GemmPar
       if (p.a_rows > 0) arow = arow < 0 ? 0 : (arow >= p.a_rows ? p.a_rows - 1 : arow);
     }
     const uint8_t *ap = p.a + arow * p.k * ELT;
-    const uint8_t *bp = p.b + (static_cast<int64_t>(e) * p.n + n) * p.k * ELT;
+    const uint8_t *bp = p.b[g] + (static_cast<int64_t>(e) * p.n + n) * p.k * ELT;
     float acc = 0.f;
     for (int kk = 0; kk < p.k; ++kk) {
       float av, bv;
@@ -59,28 +59,28 @@ __global__ __launch_bounds__(256) void grouped_gemm_generic_kernel(const GemmPar
       }
       acc = fmaf(av, bv, acc);
     }
-    float v = acc * scalar * (p.alpha ? p.alpha[e] : 1.f) * (p.row_scale ? p.row_scale[r] : 1.f);
+    float v = acc * scalar * (p.alpha[g] ? p.alpha[g][e] : 1.f) * (p.row_scale ? p.row_scale[r] : 1.f);
     if (p.col_scale) v *= p.col_scale[static_cast<int64_t>(e) * p.n + n];
     int64_t drow = r;
     if (p.scatter_d) {
       drow = p.scatter_d[r];
       if (drow < 0 || drow >= p.max_rows) continue;
     }
-    if (p.d_fp32) static_cast<float *>(p.d)[drow * p.n + n] = v;
-    else static_cast<uint16_t *>(p.d)[drow * p.n + n] = float_to_bf16_bits(v);
+    if (p.d_fp32) static_cast<float *>(p.d[g])[drow * p.n + n] = v;
+    else static_cast<uint16_t *>(p.d[g])[drow * p.n + n] = float_to_bf16_bits(v);
   }
 }
 
 // Shapes the MFMA kernel takes: K a multiple of 64 bytes, N a multiple of 4, aligned pointers, and
 // operands its 32-bit buffer offsets can span (a gathered A as a whole, 256 rows of an ungathered A, one
 // expert's weights).  Everything else runs the generic kernel.
-bool mfma_path_ok(const fluxmi_grouped_gemm_args *a) {
+bool mfma_path_ok(const fluxmi_grouped_gemm_args *a, const void *b, const void *d) {
   const int elt = a->dtype == FLUXMI_BF16 ? 2 : 1;
   const int64_t kbytes = static_cast<int64_t>(a->k) * elt;
   const int64_t span = 0xffffffffll;
   const bool a_fits = a->gather_a ? (a->a_rows > 0 && a->a_rows * kbytes <= span) : BM * kbytes <= span;
   return kbytes % KBYTES == 0 && kbytes >= KBYTES && a->n % 4 == 0 && aligned16(a->a) &&
-         aligned16(a->b) && (reinterpret_cast<uintptr_t>(a->d) & (a->d_fp32 ? 15u : 7u)) == 0 &&
+         aligned16(b) && (reinterpret_cast<uintptr_t>(d) & (a->d_fp32 ? 15u : 7u)) == 0 &&
          (a->col_scale == nullptr || aligned16(a->col_scale)) && a_fits && a->n * kbytes <= span;
 }
 
@@ -89,8 +89,11 @@ bool mfma_path_ok(const fluxmi_grouped_gemm_args *a) {
 
 extern "C" size_t fluxmi_grouped_gemm_workspace_bytes(const fluxmi_grouped_gemm_args *) { return 0; }
 
-extern "C" int fluxmi_grouped_gemm(const fluxmi_grouped_gemm_args *args, void *, size_t, void *stream) {
-  using namespace fluxmi;
+namespace fluxmi {
+namespace {
+
+int run_grouped_gemm(const fluxmi_grouped_gemm_args *args, int ngroups, const void *const *b, void *const *d,
+                     const float *const *alpha, void *stream) {
   FLUXMI_REQUIRE(args != nullptr, FLUXMI_ERR_INVALID_ARG, "grouped_gemm: null args");
   FLUXMI_REQUIRE(args->dtype == FLUXMI_BF16 || args->dtype == FLUXMI_FP8_E4M3, FLUXMI_ERR_INVALID_ARG,
                  "grouped_gemm: unknown dtype %d", args->dtype);
@@ -102,19 +105,28 @@ extern "C" int fluxmi_grouped_gemm(const fluxmi_grouped_gemm_args *args, void *,
   FLUXMI_REQUIRE(args->max_rows >= 0 && args->n >= 0 && args->k >= 0, FLUXMI_ERR_INVALID_ARG,
                  "grouped_gemm: negative size (max_rows=%d, n=%d, k=%d)", args->max_rows, args->n,
                  args->k);
+  FLUXMI_REQUIRE(ngroups >= 1 && ngroups <= kMaxWeightGroups, FLUXMI_ERR_UNSUPPORTED,
+                 "grouped_gemm: ngroups=%d outside [1,%d]", ngroups, kMaxWeightGroups);
   if (args->max_rows == 0 || args->n == 0) return FLUXMI_OK;
   FLUXMI_REQUIRE(args->k >= 1, FLUXMI_ERR_UNSUPPORTED, "grouped_gemm: k must be positive");
-  FLUXMI_REQUIRE(args->a && args->b && args->d && args->splits, FLUXMI_ERR_INVALID_ARG,
-                 "grouped_gemm: null a / b / d / splits");
+  FLUXMI_REQUIRE(args->a && args->splits && b && d, FLUXMI_ERR_INVALID_ARG, "grouped_gemm: null a / b / d / splits");
 
   GemmParams p;
+  bool mfma = true;
+  for (int g = 0; g < kMaxWeightGroups; ++g) {
+    const int src = g < ngroups ? g : 0;
+    FLUXMI_REQUIRE(b[src] && d[src], FLUXMI_ERR_INVALID_ARG, "grouped_gemm: null b / d of weight group %d", src);
+    p.b[g] = static_cast<const uint8_t *>(b[src]);
+    p.d[g] = d[src];
+    p.alpha[g] = alpha ? alpha[src] : nullptr;
+    mfma = mfma && mfma_path_ok(args, b[src], d[src]);
+  }
+  // The tile schedule numbers the column tiles of all groups with one int.
+  mfma = mfma && (static_cast<int64_t>(args->n) + BN) * ngroups < (1ll << 30);
   p.a = static_cast<const uint8_t *>(args->a);
-  p.b = static_cast<const uint8_t *>(args->b);
-  p.d = args->d;
   p.splits = args->splits;
   p.gather_a = args->gather_a;
   p.scatter_d = args->scatter_d;
-  p.alpha = args->alpha;
   p.row_scale = args->row_scale;
   p.col_scale = args->col_scale;
   p.scalar_dev = args->scalar_scale_dev;
@@ -125,25 +137,44 @@ extern "C" int fluxmi_grouped_gemm(const fluxmi_grouped_gemm_args *args, void *,
   p.n = args->n;
   p.k = args->k;
   p.d_fp32 = args->d_fp32;
+  p.ngroups = ngroups;
 
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int cus = fluxmi_device_cu_count();
   FLUXMI_REQUIRE(cus > 0, FLUXMI_ERR_HIP, "grouped_gemm: cannot query the device");
 
-  if (mfma_path_ok(args)) {
+  if (mfma) {
     // Upper bound of the tile count: never launch more workgroups than tiles.
-    const int64_t tiles_n = (args->n + BN - 1) / BN;
+    const int64_t tiles_n = (args->n + BN - 1) / BN * ngroups;
     const int64_t max_tiles = (static_cast<int64_t>(args->max_rows) / BM + args->nexperts) * tiles_n;
     const int grid = static_cast<int>(max_tiles < cus ? max_tiles : cus);
     const int rc = args->dtype == FLUXMI_BF16 ? launch_grouped_gemm_bf16(p, grid, s) : launch_grouped_gemm_fp8(p, grid, s);
     if (rc != FLUXMI_OK) return rc;
   } else {
     const int grid = cus * 8;
-    if (args->dtype == FLUXMI_BF16)
-      hipLaunchKernelGGL(grouped_gemm_generic_kernel<2>, dim3(grid), dim3(256), 0, s, p);
-    else
-      hipLaunchKernelGGL(grouped_gemm_generic_kernel<1>, dim3(grid), dim3(256), 0, s, p);
+    for (int g = 0; g < ngroups; ++g) {
+      if (args->dtype == FLUXMI_BF16)
+        hipLaunchKernelGGL(grouped_gemm_generic_kernel<2>, dim3(grid), dim3(256), 0, s, p, g);
+      else
+        hipLaunchKernelGGL(grouped_gemm_generic_kernel<1>, dim3(grid), dim3(256), 0, s, p, g);
+    }
   }
   FLUXMI_HIP_CHECK(hipGetLastError());
   return FLUXMI_OK;
+}
+
+}  // namespace
+}  // namespace fluxmi
+
+extern "C" int fluxmi_grouped_gemm(const fluxmi_grouped_gemm_args *args, void *, size_t, void *stream) {
+  FLUXMI_REQUIRE(args != nullptr, FLUXMI_ERR_INVALID_ARG, "grouped_gemm: null args");
+  const void *b = args->b;
+  void *d = args->d;
+  const float *alpha = args->alpha;
+  return fluxmi::run_grouped_gemm(args, 1, &b, &d, &alpha, stream);
+}
+
+extern "C" int fluxmi_grouped_gemm_multi(const fluxmi_grouped_gemm_args *args, int32_t ngroups, const void *const *b,
+                                         void *const *d, const float *const *alpha, void *, size_t, void *stream) {
+  return fluxmi::run_grouped_gemm(args, ngroups, b, d, alpha, stream);
 }

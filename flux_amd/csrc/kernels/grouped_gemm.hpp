@@ -54,14 +54,17 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
+constexpr int kMaxWeightGroups = 4;
+
+// b / d / alpha: one entry per weight group of the launch (the same rows times several weight tensors).
 struct GemmParams {
   const uint8_t *a;
-  const uint8_t *b;
-  void *d;
+  const uint8_t *b[kMaxWeightGroups];
+  void *d[kMaxWeightGroups];
   const int32_t *splits;
   const int32_t *gather_a;
   const int32_t *scatter_d;
-  const float *alpha;
+  const float *alpha[kMaxWeightGroups];
   const float *row_scale;
   const float *col_scale;
   const float *scalar_dev;
@@ -72,6 +75,7 @@ struct GemmParams {
   int32_t n;
   int32_t k;
   int32_t d_fp32;
+  int32_t ngroups;
 };
 
 

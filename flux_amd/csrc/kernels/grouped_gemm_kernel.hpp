@@ -111,8 +111,8 @@ __device__ __forceinline__ float acc_read(float a) {
 // scatter), so no store is predicated.  OUT_F32 selects the output element type.  !SCALED: every scale
 // factor is 1 and the multiplications are left out.
 template <int ELT, int MB, int NB, bool FULL, bool OUT_F32, bool SCALED>
-__device__ __forceinline__ void store_tile(uint8_t *windows, const TileCtx &c, int e, int row_base, int rows_e, int wrow0,
-                                           int wcol0,
+__device__ __forceinline__ void store_tile(uint8_t *windows, const TileCtx &c, int g, int e, int row_base, int rows_e,
+                                           int wrow0, int wcol0,
                                            const typename Geom<ELT>::Acc (&acc)[32 * MB / Geom<ELT>::BLK][32 * NB / Geom<ELT>::BLK]) {
   static_assert(MB % 2 == 0, "a window holds 64 rows");
   constexpr int BLK = Geom<ELT>::BLK;
@@ -122,7 +122,7 @@ __device__ __forceinline__ void store_tile(uint8_t *windows, const TileCtx &c, i
   const int lane = c.lane;
   const int h = lane >> 5;
   const int n = p->n;
-  const float *alpha = p->alpha, *row_scale = p->row_scale, *col_scale = p->col_scale;
+  const float *alpha = p->alpha[g], *row_scale = p->row_scale, *col_scale = p->col_scale;
   const float tile_scale = c.scalar * (alpha ? alpha[e] : 1.f);
   float rs[MBK];  // scale of this lane's row in each block row
 #pragma unroll
@@ -134,7 +134,7 @@ __device__ __forceinline__ void store_tile(uint8_t *windows, const TileCtx &c, i
   const int cc = lane & 7;    // its 4-column chunk
   // Output address of (first row of the wave + rr0, first column of the wave + 4 * cc); blocks and row
   // groups add multiples of 32 columns and 8 rows.
-  uint8_t *const d = static_cast<uint8_t *>(p->d);
+  uint8_t *const d = static_cast<uint8_t *>(p->d[g]);
   uint8_t *dlane = d + (static_cast<int64_t>(row_base + wrow0 + rr0) * n + wcol0 + cc * 4) * ELT_OUT;
   const int64_t rowgroup_bytes = static_cast<int64_t>(8) * n * ELT_OUT;
   const int32_t *scatter = FULL ? nullptr : p->scatter_d;
@@ -218,9 +218,25 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const uint8_t *base,
 }
 // Where a work item lies.  kind: 0 a whole macro tile (4, 4); 1 the 128-row tile ending an expert (2, 4);
 // 2 a 256x128 piece (4, 2); 3 a 128x128 piece (2, 2); -1 an item without work; -2 past the last item.
+// n0 is a column of the launch's virtual output: weight group g (a launch may multiply the same rows by up
+// to four weight tensors, each with an output of its own) occupies columns [g * npad, g * npad + n), npad =
+// n rounded up to whole macro tiles.
 struct TileDesc {
   int kind, e, row_base, rows_e, m0, n0;
 };
+
+// Virtual column -> weight group (returned) and column inside it (n0).
+__device__ __forceinline__ int split_group(int &n0, int n, int ngroups) {
+  int g = 0;
+  if (ngroups > 1) {
+    const int npad = ((n + BN - 1) / BN) * BN;
+    while (n0 >= npad) {
+      n0 -= npad;
+      ++g;
+    }
+  }
+  return g;
+}
 
 // Ring geometry per tile shape.  Whole and half tiles: five stages of 32 KiB, fills four k-steps ahead.  The
 // 128x128 pieces of a last round need 16 KiB per stage and have short k-steps (16 MFMAs per wave), so four
@@ -260,7 +276,9 @@ __device__ __forceinline__ void setup_operands(const GemmParams &p, const TileCt
   const uint8_t *xbase = gathered ? p.a : p.a + static_cast<int64_t>(t.row_base + t.m0) * c.kbytes;
   const int64_t xrows = gathered ? p.a_rows : t.rows_e - t.m0;
   op.xrsrc = make_rsrc(xbase, xrows > 0 ? xrows * c.kbytes : 0xffffffffll);
-  op.wrsrc = make_rsrc(p.b + (static_cast<int64_t>(t.e) * p.n + t.n0) * c.kbytes, static_cast<int64_t>(p.n - t.n0) * c.kbytes);
+  int n0 = t.n0;
+  const int g = split_group(n0, p.n, p.ngroups);
+  op.wrsrc = make_rsrc(kernel_args()->b[g] + (static_cast<int64_t>(t.e) * p.n + n0) * c.kbytes, static_cast<int64_t>(p.n - n0) * c.kbytes);
 #pragma unroll
   for (int j = 0; j < XL; ++j) {
     int xr = t.m0 + (XL * c.wave + j) * 16 + c.fill_row;
@@ -274,9 +292,9 @@ __device__ __forceinline__ void setup_operands(const GemmParams &p, const TileCt
   }
 #pragma unroll
   for (int j = 0; j < WL; ++j) {
-    int wr = t.n0 + (WL * c.wave + j) * 16 + c.fill_row;
+    int wr = n0 + (WL * c.wave + j) * 16 + c.fill_row;
     if (wr > p.n - 1) wr = p.n - 1;
-    op.woff[j] = static_cast<uint32_t>((wr - t.n0) * c.kbytes) + c.fill_chunk * 16;
+    op.woff[j] = static_cast<uint32_t>((wr - n0) * c.kbytes) + c.fill_chunk * 16;
   }
 }
 
@@ -330,7 +348,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
   constexpr int NM = MBK * NBK;          // MFMAs per k-step
   constexpr int RSPAN = NM / 2;        // MFMA slots over which the fragment reads of a step are spread
   const int wave = c.wave, lane = c.lane, wm = c.wm, wn = c.wn, nk = c.nk;
-  const int e = t.e, row_base = t.row_base, rows_e = t.rows_e, m0 = t.m0, n0 = t.n0;
+  const int e = t.e, row_base = t.row_base, rows_e = t.rows_e, m0 = t.m0;
 
   // Operand addressing: prepared by the previous tile together with the first fills, or set up here.
   bool prefetched = false;
@@ -561,21 +579,23 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
   }
   uint8_t *windows = smem + 4 * STAGE_BYTES + wave * 8192;  // one 8 KiB window per wave
   const int wrow0 = m0 + wm * (32 * MB);
-  const int wcol0 = n0 + wn * (32 * NB);
   {
     const KernArgs pe = kernel_args();
+    int n0 = t.n0;
+    const int g = split_group(n0, pe->n, pe->ngroups);
+    const int wcol0 = n0 + wn * (32 * NB);
     const bool full = wrow0 + 32 * MB <= rows_e && wcol0 + 32 * NB <= pe->n && pe->scatter_d == nullptr;
     const bool out_f32 = pe->d_fp32 != 0;
-    const bool scaled = !(c.scalar == 1.f && pe->alpha == nullptr && pe->row_scale == nullptr && pe->col_scale == nullptr);
+    const bool scaled = !(c.scalar == 1.f && pe->alpha[g] == nullptr && pe->row_scale == nullptr && pe->col_scale == nullptr);
     if (full && !scaled) {
-      if (out_f32) store_tile<ELT, MB, NB, true, true, false>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
-      else store_tile<ELT, MB, NB, true, false, false>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
+      if (out_f32) store_tile<ELT, MB, NB, true, true, false>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, acc);
+      else store_tile<ELT, MB, NB, true, false, false>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, acc);
     } else if (full) {
-      if (out_f32) store_tile<ELT, MB, NB, true, true, true>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
-      else store_tile<ELT, MB, NB, true, false, true>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
+      if (out_f32) store_tile<ELT, MB, NB, true, true, true>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, acc);
+      else store_tile<ELT, MB, NB, true, false, true>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, acc);
     } else {
-      if (out_f32) store_tile<ELT, MB, NB, false, true, true>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
-      else store_tile<ELT, MB, NB, false, false, true>(windows, c, e, row_base, rows_e, wrow0, wcol0, acc);
+      if (out_f32) store_tile<ELT, MB, NB, false, true, true>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, acc);
+      else store_tile<ELT, MB, NB, false, false, true>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, acc);
     }
   }
   __builtin_amdgcn_s_barrier();  // the LDS windows are free again before the next tile's fills start
@@ -592,7 +612,8 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
   c.wn = c.wave & 1;   // column half
   c.wm = c.wave >> 1;  // row half
   const int lane = c.lane;
-  const int tiles_n = (p.n + BN - 1) / BN;
+  const int tiles_n1 = (p.n + BN - 1) / BN;  // column tiles of one weight group
+  const int tiles_n = tiles_n1 * p.ngroups;  // ... of the launch
   c.kbytes = static_cast<int64_t>(p.k) * ELT;
   c.nk = static_cast<int>(c.kbytes / KBYTES);
 
@@ -702,7 +723,9 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
     t.row_base = row_base;
     t.rows_e = rows_e;
     t.m0 = mt * BM;
-    t.n0 = nt * BN;
+    const int g = p.ngroups > 1 ? nt / tiles_n1 : 0;
+    const int gcol = g * tiles_n1 * BN;  // first virtual column of the weight group
+    t.n0 = (nt - g * tiles_n1) * BN;
     if (item < full_items || pieces == 1) {
       // The last row tile of an expert is run 128 rows high when that covers its rows.
       t.kind = rows_e - t.m0 > 128 ? 0 : 1;
@@ -714,6 +737,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
       t.n0 += (piece & 1) * 128;
       t.kind = (t.m0 < rows_e && t.n0 < p.n) ? 3 : -1;
     }
+    t.n0 += gcol;
     return t;
   };
 

@@ -5,6 +5,7 @@
 // Same constructor and method signatures, same argument checks; every launch goes to the current HIP
 // stream and nothing synchronises the host (the reference's layer0 blocks once to read the splits back,
 // gemm_grouped_v3_ag_scatter.cc:323-331 — here the tile schedule is built on the device).
+#include <algorithm>
 #include <cstdlib>
 
 #include "ths_ops.h"
@@ -110,10 +111,34 @@ std::vector<torch::Tensor> GemmGroupedV3AGScatter::forward_impl(
                                          moe_args_.topk, gather_index_.data_ptr<int32_t>(), nullptr,
                                          current_stream()),
                  "fluxmi_moe_gather_index");
-    for (size_t i = 0; i < groups; ++i) {
-      const float *alpha = output_scale.has_value() ? output_scale->at(i).data_ptr<float>() : nullptr;
-      run_grouped_gemm(inputs_shard, weights[i], splits_gpu, outputs[i], gather_index_.data_ptr<int32_t>(),
-                       nrows, alpha, nullptr, nullptr, nullptr);
+    // All weight groups (gate and up projections, say) run as one launch over one tile schedule: the
+    // gathered A tiles an XCD's L2 holds serve every group, and the launch has one tail instead of one per
+    // group (the reference shares the gathered A the same way, gemm_grouped_v3_ag_scatter.cc:375-395).
+    constexpr size_t kMaxGroupsPerLaunch = 4;
+    for (size_t g0 = 0; g0 < groups; g0 += kMaxGroupsPerLaunch) {
+      const size_t ng = std::min(kMaxGroupsPerLaunch, groups - g0);
+      const void *b[kMaxGroupsPerLaunch];
+      void *d[kMaxGroupsPerLaunch];
+      const float *alpha[kMaxGroupsPerLaunch];
+      for (size_t i = 0; i < ng; ++i) {
+        b[i] = weights[g0 + i].data_ptr();
+        d[i] = outputs[g0 + i].data_ptr();
+        alpha[i] = output_scale.has_value() ? output_scale->at(g0 + i).data_ptr<float>() : nullptr;
+      }
+      fluxmi_grouped_gemm_args args{};
+      args.dtype = to_fluxmi_dtype(inputs_shard.scalar_type());
+      args.nexperts = static_cast<int32_t>(moe_args_.nexperts);
+      args.max_rows = static_cast<int32_t>(nrows);
+      args.n = static_cast<int32_t>(moe_args_.ffn_hidden);
+      args.k = static_cast<int32_t>(moe_args_.hidden);
+      args.a_rows = static_cast<int32_t>(ntokens);
+      args.a = inputs_shard.data_ptr();
+      args.splits = splits_gpu.data_ptr<int32_t>();
+      args.gather_a = gather_index_.data_ptr<int32_t>();
+      args.scalar_scale = 1.0f;
+      check_status(fluxmi_grouped_gemm_multi(&args, static_cast<int32_t>(ng), b, d, alpha, nullptr, 0,
+                                             current_stream()),
+                   "fluxmi_grouped_gemm_multi");
     }
   }
   if (allgather_output.has_value()) {  // gemm_grouped_v3_ag_scatter.cc:440-445

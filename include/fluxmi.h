@@ -112,6 +112,16 @@ size_t fluxmi_grouped_gemm_workspace_bytes(const fluxmi_grouped_gemm_args *args)
 int fluxmi_grouped_gemm(const fluxmi_grouped_gemm_args *args, void *workspace,
                         size_t workspace_bytes, void *stream);
 
+/* The same rows times `ngroups` (1..4) weight tensors in ONE launch, each group with an output of its own:
+ * `GemmGroupedV3AGScatterOp::forward_multiple_weights` (gate and up projections sharing the gathered
+ * A tiles; src/moe_ag_scatter/ths_op/gemm_grouped_v3_ag_scatter.cc:375-395).  b, d and alpha are
+ * HOST arrays of `ngroups` device pointers (alpha itself, or single entries of it, may be NULL); the b, d
+ * and alpha members of `args` are ignored, every other member is shared by all groups.  The column tiles
+ * of all groups form one tile schedule, so the tail of the launch is shared as well. */
+int fluxmi_grouped_gemm_multi(const fluxmi_grouped_gemm_args *args, int32_t ngroups, const void *const *b,
+                              void *const *d, const float *const *alpha, void *workspace,
+                              size_t workspace_bytes, void *stream);
+
 /* ------------------------------------------------------------------------------------------------
  * Top-k (weighted) gather-reduce back to token order (the reduce half of layer1).
  *

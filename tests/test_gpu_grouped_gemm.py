@@ -70,6 +70,47 @@ def test_bf16_gather_scatter_and_scales():
     assert_close(out, ref_scattered, "gather+scatter+scales")
 
 
+@pytest.mark.parametrize("ngroups,experts,tokens,topk,h,n,seed,scaled", [
+    (2, 4, 500, 2, 256, 520, 0, True),      # N not a whole number of macro tiles: the groups' column ranges are padded
+    (3, 6, 300, 3, 320, 256, 1, False),
+    (4, 2, 64, 1, 64, 8, 2, True),
+    (2, 8, 4096, 2, 512, 1024, 3, True),    # 144 + tiles on 256 CUs: the last round is cut into pieces
+    (2, 3, 40, 2, 72, 50, 4, True),         # K and N of the generic kernel
+])
+def test_bf16_multiple_weight_groups_one_launch(ngroups, experts, tokens, topk, h, n, seed, scaled):
+    """forward_multiple_weights' kernel form: the same gathered rows times several weight tensors in one
+    launch must equal one launch per weight tensor, and the oracle."""
+    from flux_amd import capi
+    print(f"[case] grouped_gemm_multi groups={ngroups} E={experts} T={tokens} k={topk} H={h} N={n}", flush=True)
+    rng = np.random.default_rng(100 + seed)
+    g = torch.Generator().manual_seed(100 + seed)
+    choosed = np.stack([rng.permutation(experts)[:topk] for _ in range(tokens)]).astype(np.int32)
+    split = routing.splits(choosed, experts)
+    gi, _ = routing.gather_index(routing.scatter_index_stable(choosed, experts), topk)
+    x = torch.randn(tokens, h, generator=g).to(torch.bfloat16)
+    ws = [(torch.randn(experts, n, h, generator=g) * 0.05).to(torch.bfloat16) for _ in range(ngroups)]
+    alphas = [torch.rand(experts, generator=g) + 0.5 if (scaled and i != 1) else None for i in range(ngroups)]
+    xs = x[torch.as_tensor(gi, dtype=torch.long)]
+    sp, gd, xd = torch.from_numpy(split).cuda(), torch.from_numpy(gi).cuda(), x.cuda()
+    outs = capi.grouped_gemm_multi(xd, [w.cuda() for w in ws], sp, gather_a=gd,
+                                   alphas=[None if al is None else al.cuda() for al in alphas] if scaled else None)
+    assert len(outs) == ngroups
+    for i in range(ngroups):
+        ref = layers.grouped_gemm_fp32(xs, ws[i], split, alpha=alphas[i])
+        assert_close(outs[i], ref, f"group {i}")
+        single = capi.grouped_gemm(xd, ws[i].cuda(), sp, gather_a=gd, alpha=None if alphas[i] is None else alphas[i].cuda())
+        assert torch.equal(outs[i], single), f"group {i}: one launch for all groups differs from a launch per group"
+
+
+def test_multiple_weight_groups_argument_checks():
+    from flux_amd import capi
+    x = torch.zeros(8, 64, dtype=torch.bfloat16, device="cuda")
+    w = torch.zeros(1, 8, 64, dtype=torch.bfloat16, device="cuda")
+    sp = torch.tensor([8], dtype=torch.int32, device="cuda")
+    with pytest.raises(RuntimeError, match="ngroups"):
+        capi.grouped_gemm_multi(x, [w] * 5, sp)
+
+
 def test_bf16_generic_kernel_odd_shapes():
     """K not a multiple of 32 and N not a multiple of 4 take the generic kernel."""
     from flux_amd import capi
@@ -248,3 +289,21 @@ def test_fp8_benchmark_c5_layer1():
             ref1[i] += float(wl.row_weight[r]) * float(sa[r]) * ((qa[r].float() @ qw[e].float().t()) * sw[e])
     got = out[torch.as_tensor(tok).cuda()].float().cpu()
     assert float((got - ref1).norm() / ref1.norm()) < FP8_FROB
+
+
+def test_fp8_multiple_weight_groups_one_launch():
+    from flux_amd import capi
+    g = torch.Generator().manual_seed(77)
+    experts, rows, n, k = 4, 1000, 384, 256
+    split = random_splits(np.random.default_rng(77), experts, rows)
+    a8 = torch.randn(rows, k, generator=g).to(torch.float8_e4m3fn)
+    ws = [torch.randn(experts, n, k, generator=g).to(torch.float8_e4m3fn) for _ in range(2)]
+    rs = torch.rand(rows, generator=g) + 0.5
+    sp = torch.from_numpy(split).cuda()
+    outs = capi.grouped_gemm_multi(a8.cuda(), [w.cuda() for w in ws], sp, row_scale=rs.cuda())
+    for i in range(2):
+        single = capi.grouped_gemm(a8.cuda(), ws[i].cuda(), sp, row_scale=rs.cuda())
+        assert torch.equal(outs[i], single)
+        ref = layers.grouped_gemm_fp32(a8.float(), ws[i].float(), split, row_scale=rs)
+        err = (outs[i].float().cpu() - ref).norm() / ref.norm()
+        assert float(err) < FP8_FROB
