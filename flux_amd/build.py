@@ -105,6 +105,7 @@ def build_ths_op(force=True):
     _run([
         "g++", "-shared", *objs, "-o", out, f"-L{torch_lib}", f"-L{LIB_DIR}",
         "-ltorch", "-ltorch_cpu", "-ltorch_hip", "-ltorch_python", "-lc10", "-lc10_hip", "-lfluxmi_kernels",
+        "-L/opt/rocm/lib", "-lamdhip64",
         "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{torch_lib}",
     ])
     return out

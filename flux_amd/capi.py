@@ -33,6 +33,8 @@ class GroupedGemmArgs(ctypes.Structure):
         ("alpha", ctypes.c_void_p), ("row_scale", ctypes.c_void_p), ("col_scale", ctypes.c_void_p),
         ("scalar_scale", ctypes.c_float), ("d_fp32", ctypes.c_int32),
         ("scalar_scale_dev", ctypes.c_void_p),
+        ("cu_margin", ctypes.c_int32), ("raster_rows", ctypes.c_int32), ("sched_flags", ctypes.c_int32),
+        ("reserved", ctypes.c_int32),
     ]
 
 
@@ -120,8 +122,13 @@ def gather_index(scatter_index, topk):
     return gather, tki
 
 
+SCHED_WHOLE_TAIL_TILES = 1
+SCHED_NO_HALF_TILES = 2
+
+
 def grouped_gemm(a, b, splits, out=None, gather_a=None, scatter_d=None, alpha=None, row_scale=None,
-                 col_scale=None, scalar_scale=1.0, scalar_scale_dev=None, max_rows=None, out_dtype=None):
+                 col_scale=None, scalar_scale=1.0, scalar_scale_dev=None, max_rows=None, out_dtype=None,
+                 cu_margin=0, raster_rows=0, sched_flags=0):
     """D = grouped GEMM of A [rows_a, K] with B [E, N, K]; see fluxmi_grouped_gemm in include/fluxmi.h."""
     lib = load()
     if a.dtype == torch.bfloat16:
@@ -159,7 +166,8 @@ def grouped_gemm(a, b, splits, out=None, gather_a=None, scatter_d=None, alpha=No
         row_scale=None if row_scale is None else row_scale.data_ptr(),
         col_scale=None if col_scale is None else col_scale.data_ptr(),
         scalar_scale=float(scalar_scale), d_fp32=int(out.dtype == torch.float32),
-        scalar_scale_dev=None if scalar_scale_dev is None else scalar_scale_dev.data_ptr())
+        scalar_scale_dev=None if scalar_scale_dev is None else scalar_scale_dev.data_ptr(),
+        cu_margin=cu_margin, raster_rows=raster_rows, sched_flags=sched_flags)
     _check(lib.fluxmi_grouped_gemm(ctypes.byref(args), None, 0, _stream()), "fluxmi_grouped_gemm")
     return out
 

@@ -138,10 +138,19 @@ int run_grouped_gemm(const fluxmi_grouped_gemm_args *args, int ngroups, const vo
   p.k = args->k;
   p.d_fp32 = args->d_fp32;
   p.ngroups = ngroups;
+  FLUXMI_REQUIRE(args->raster_rows >= 0 && args->raster_rows <= 1024, FLUXMI_ERR_INVALID_ARG,
+                 "grouped_gemm: raster_rows=%d outside [0,1024]", args->raster_rows);
+  FLUXMI_REQUIRE(args->cu_margin >= 0, FLUXMI_ERR_INVALID_ARG, "grouped_gemm: negative cu_margin");
+  FLUXMI_REQUIRE((args->sched_flags & ~(FLUXMI_SCHED_WHOLE_TAIL_TILES | FLUXMI_SCHED_NO_HALF_TILES)) == 0,
+                 FLUXMI_ERR_INVALID_ARG, "grouped_gemm: unknown sched_flags 0x%x", args->sched_flags);
+  p.raster_rows = args->raster_rows > 0 ? args->raster_rows : 8;
+  p.sched_flags = args->sched_flags;
 
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const int cus = fluxmi_device_cu_count();
+  int cus = fluxmi_device_cu_count();
   FLUXMI_REQUIRE(cus > 0, FLUXMI_ERR_HIP, "grouped_gemm: cannot query the device");
+  // CUs left to other work of the caller (Flux's sm_margin): the persistent kernel launches fewer workgroups.
+  cus = cus - args->cu_margin > 1 ? cus - args->cu_margin : 1;
 
   if (mfma) {
     // Upper bound of the tile count: never launch more workgroups than tiles.

@@ -76,6 +76,8 @@ struct GemmParams {
   int32_t k;
   int32_t d_fp32;
   int32_t ngroups;
+  int32_t raster_rows;  // row tiles per raster group, >= 1
+  int32_t sched_flags;  // FLUXMI_SCHED_*
 };
 
 

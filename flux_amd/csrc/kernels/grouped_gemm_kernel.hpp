@@ -675,7 +675,9 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
   // chip does not idle while a fraction of the CUs finishes whole tiles.
   const int full_items = (total_tiles / grid) * grid;
   const int rem_tiles = total_tiles - full_items;
-  const int pieces = rem_tiles * 4 <= grid ? 4 : (rem_tiles * 2 <= grid ? 2 : 1);
+  const bool cut_tail = (p.sched_flags & FLUXMI_SCHED_WHOLE_TAIL_TILES) == 0;
+  const bool half_tiles = (p.sched_flags & FLUXMI_SCHED_NO_HALF_TILES) == 0;
+  const int pieces = !cut_tail ? 1 : (rem_tiles * 4 <= grid ? 4 : (rem_tiles * 2 <= grid ? 2 : 1));
   const int total_items = full_items + rem_tiles * pieces;
 
   // ---- schedule: walk the experts once, in step with this workgroup's increasing tile ids ----------
@@ -705,13 +707,13 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
       }
     }
     if (e >= p.nexperts) return t;
-    // Order inside an expert: row tiles are cut into groups of at most 8; a group is walked
+    // Order inside an expert: row tiles are cut into groups of at most p.raster_rows (8 unless tuned); a group is walked
     // column-major over all weight panels before the next group starts.  32 consecutive tiles (one
     // XCD's share of a round) then cover about 8 row tiles x 4 panels: 12 distinct operand tiles per
     // k-step for 32 CUs.
     const int m_tiles = (rows_e + BM - 1) / BM;
-    const int ngroups_m = (m_tiles + 7) >> 3;
-    const int gm = (m_tiles + ngroups_m - 1) / ngroups_m;  // group height, <= 8
+    const int ngroups_m = (m_tiles + p.raster_rows - 1) / p.raster_rows;
+    const int gm = (m_tiles + ngroups_m - 1) / ngroups_m;  // group height, <= raster_rows
     const int local = tile - tile_base;
     const int group = local / (gm * tiles_n);
     const int group_first = group * gm;
@@ -728,7 +730,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
     t.n0 = (nt - g * tiles_n1) * BN;
     if (item < full_items || pieces == 1) {
       // The last row tile of an expert is run 128 rows high when that covers its rows.
-      t.kind = rows_e - t.m0 > 128 ? 0 : 1;
+      t.kind = (rows_e - t.m0 > 128 || !half_tiles) ? 0 : 1;
     } else if (pieces == 2) {
       t.n0 += piece * 128;
       t.kind = t.n0 < p.n ? 2 : -1;

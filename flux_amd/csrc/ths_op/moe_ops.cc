@@ -8,13 +8,87 @@
 #include <algorithm>
 #include <cstdlib>
 
+#include <hip/hip_runtime_api.h>
+
 #include "ths_ops.h"
 
 namespace flux_amd {
 
+namespace {
+// Schedule forced on every launch of this thread while a profiler tries it.
+thread_local const GemmLaunchTuning *t_tuning_override = nullptr;
+
+struct ScopedTuningOverride {
+  explicit ScopedTuningOverride(const GemmLaunchTuning *t) { t_tuning_override = t; }
+  ~ScopedTuningOverride() { t_tuning_override = nullptr; }
+};
+
+GemmShapeKey shape_key(const fluxmi_grouped_gemm_args &args, int32_t ngroups) {
+  GemmShapeKey key;
+  key.dtype = args.dtype;
+  key.nexperts = args.nexperts;
+  key.n = args.n;
+  key.k = args.k;
+  key.max_rows = args.max_rows;
+  key.ngroups = ngroups;
+  return key;
+}
+
+#define FLUX_AMD_HIP_CHECK(expr)                                                                          \
+  do {                                                                                                    \
+    const hipError_t err_ = (expr);                                                                       \
+    if (err_ != hipSuccess) throw std::runtime_error(std::string(#expr " failed: ") + hipGetErrorString(err_)); \
+  } while (0)
+
+// Times `run` (one whole forward) under every candidate schedule on the current stream, 5 warm-up and 10
+// timed calls each like the reference's profiling loops (gemm_grouped_v3_ag_scatter.cc:540-590), records
+// them in `ctx` and registers the fastest for `key`.
+template <class F>
+void profile_schedules(const GemmShapeKey &key, ProfilingContext *ctx, F &&run) {
+  constexpr int kWarmIters = 5, kIters = 10;
+  hipStream_t stream = static_cast<hipStream_t>(current_stream());
+  hipEvent_t e0, e1;
+  FLUX_AMD_HIP_CHECK(hipEventCreate(&e0));
+  FLUX_AMD_HIP_CHECK(hipEventCreate(&e1));
+  try {
+    for (const GemmLaunchTuning &cand : gemm_tuning_candidates()) {
+      ScopedTuningOverride scope(&cand);
+      for (int i = 0; i < kWarmIters; ++i) run();
+      FLUX_AMD_HIP_CHECK(hipEventRecord(e0, stream));
+      for (int i = 0; i < kIters; ++i) run();
+      FLUX_AMD_HIP_CHECK(hipEventRecord(e1, stream));
+      FLUX_AMD_HIP_CHECK(hipEventSynchronize(e1));
+      float ms = 0.f;
+      FLUX_AMD_HIP_CHECK(hipEventElapsedTime(&ms, e0, e1));
+      ctx->add(key, cand, ms / kIters);
+    }
+  } catch (...) {
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    throw;
+  }
+  FLUX_AMD_HIP_CHECK(hipEventDestroy(e0));
+  FLUX_AMD_HIP_CHECK(hipEventDestroy(e1));
+  TuningTable::instance().add(key, ctx->record_best(key));
+}
+}  // namespace
+
+void apply_launch_tuning(fluxmi_grouped_gemm_args &args, int32_t ngroups, int64_t sm_margin) {
+  TORCH_CHECK(sm_margin >= 0 && sm_margin < (1 << 20), "sm_margin must be non-negative, got ", sm_margin);
+  args.cu_margin = static_cast<int32_t>(sm_margin);
+  if (t_tuning_override != nullptr) {
+    args.raster_rows = t_tuning_override->raster_rows;
+    args.sched_flags = t_tuning_override->sched_flags;
+  } else if (auto t = TuningTable::instance().find(shape_key(args, ngroups))) {
+    args.raster_rows = t->raster_rows;
+    args.sched_flags = t->sched_flags;
+  }
+}
+
 void run_grouped_gemm(const torch::Tensor &a, const torch::Tensor &b, const torch::Tensor &splits_dev,
                       torch::Tensor &d, const int32_t *gather_a, int64_t max_rows, const float *alpha,
-                      const float *row_scale, const float *col_scale, const float *scalar_dev) {
+                      const float *row_scale, const float *col_scale, const float *scalar_dev,
+                      int64_t sm_margin) {
   fluxmi_grouped_gemm_args args{};
   args.dtype = to_fluxmi_dtype(a.scalar_type());
   args.nexperts = static_cast<int32_t>(b.size(0));
@@ -34,6 +108,7 @@ void run_grouped_gemm(const torch::Tensor &a, const torch::Tensor &b, const torc
   args.scalar_scale = 1.0f;
   args.d_fp32 = d.scalar_type() == at::ScalarType::Float ? 1 : 0;
   args.scalar_scale_dev = scalar_dev;
+  apply_launch_tuning(args, 1, sm_margin);
   check_status(fluxmi_grouped_gemm(&args, nullptr, 0, current_stream()), "fluxmi_grouped_gemm");
 }
 
@@ -60,7 +135,7 @@ std::vector<torch::Tensor> GemmGroupedV3AGScatter::forward_impl(
     torch::Tensor inputs_shard, std::vector<torch::Tensor> weights, torch::Tensor splits_gpu,
     torch::Tensor scatter_index, std::optional<std::vector<torch::Tensor>> output_scale,
     std::optional<std::vector<torch::Tensor>> outputs_buf, std::optional<torch::Tensor> allgather_output,
-    bool /*fast_accum*/, int64_t /*sm_margin*/) {
+    bool /*fast_accum*/, int64_t sm_margin) {
   FLUX_AMD_CHECK_INPUT(inputs_shard, moe_args_.input_dtype);
   FLUX_AMD_CHECK_NDIM(inputs_shard, 2);
   const int64_t ntokens = inputs_shard.size(0);  // world size 1: the shard is the whole batch
@@ -136,6 +211,7 @@ std::vector<torch::Tensor> GemmGroupedV3AGScatter::forward_impl(
       args.splits = splits_gpu.data_ptr<int32_t>();
       args.gather_a = gather_index_.data_ptr<int32_t>();
       args.scalar_scale = 1.0f;
+      apply_launch_tuning(args, static_cast<int32_t>(ng), sm_margin);
       check_status(fluxmi_grouped_gemm_multi(&args, static_cast<int32_t>(ng), b, d, alpha, nullptr, 0,
                                              current_stream()),
                    "fluxmi_grouped_gemm_multi");
@@ -170,6 +246,30 @@ std::vector<torch::Tensor> GemmGroupedV3AGScatter::forward_multiple_weights(
                       allgather_output, fast_accum, sm_margin);
 }
 
+torch::Tensor GemmGroupedV3AGScatter::profiling(torch::Tensor inputs_shard, torch::Tensor weights,
+                                                torch::Tensor splits_gpu, torch::Tensor scatter_index,
+                                                std::optional<torch::Tensor> output_scale,
+                                                std::optional<torch::Tensor> outputs_buf,
+                                                std::optional<torch::Tensor> allgather_output, bool fast_accum,
+                                                int64_t sm_margin, std::shared_ptr<ProfilingContext> prof_ctx) {
+  ProfilingContext tmp_ctx("__tmp__");
+  ProfilingContext *ctx = prof_ctx ? prof_ctx.get() : &tmp_ctx;
+  auto run = [&]() {
+    return forward(inputs_shard, weights, splits_gpu, scatter_index, output_scale, outputs_buf, allgather_output,
+                   fast_accum, sm_margin);
+  };
+  run();  // argument checks before anything is timed
+  GemmShapeKey key;
+  key.dtype = to_fluxmi_dtype(moe_args_.input_dtype);
+  key.nexperts = moe_args_.nexperts;
+  key.n = moe_args_.ffn_hidden;
+  key.k = moe_args_.hidden;
+  key.max_rows = static_cast<int32_t>(inputs_shard.size(0) * moe_args_.topk);
+  key.ngroups = 1;
+  if (key.max_rows > 0) profile_schedules(key, ctx, run);
+  return run();  // with the schedule just registered
+}
+
 // ------------------------------------------------------------------------------------------------
 // Layer1: grouped GEMM + top-k gather-reduce
 // ------------------------------------------------------------------------------------------------
@@ -202,7 +302,7 @@ torch::Tensor GemmGroupedV3GatherRS::forward_impl(
     std::vector<torch::Tensor> inputs, std::vector<torch::Tensor> weights, torch::Tensor splits_cpu,
     torch::Tensor routing_idx, std::optional<std::vector<torch::Tensor>> input_scale,
     std::optional<std::vector<torch::Tensor>> weight_scale,
-    std::optional<std::vector<torch::Tensor>> output_vec_scale, bool with_stream_sync) {
+    std::optional<std::vector<torch::Tensor>> output_vec_scale, bool with_stream_sync, int64_t sm_margin) {
   TORCH_CHECK(!inputs.empty() && inputs.size() == weights.size(), "inputs / weights group count mismatch");
   TORCH_CHECK(static_cast<int64_t>(inputs.size()) <= max_input_groups_, "more input groups than max_input_groups");
   const at::ScalarType st = weights[0].scalar_type();
@@ -264,7 +364,7 @@ torch::Tensor GemmGroupedV3GatherRS::forward_impl(
       else TORCH_CHECK(false, "input_scale must be [1] or [M]");
     }
     if (row_holder.defined()) row = row_holder.data_ptr<float>();
-    run_grouped_gemm(inputs[g], weights[g], splits_dev_, inter_[g], nullptr, m, alpha, row, col, scalar);
+    run_grouped_gemm(inputs[g], weights[g], splits_dev_, inter_[g], nullptr, m, alpha, row, col, scalar, sm_margin);
     group_ptrs.push_back(inter_[g].data_ptr());
   }
   check_status(fluxmi_topk_gather_reduce(group_ptrs.data(), static_cast<int32_t>(groups), inter_fp32_ ? 1 : 0,
@@ -280,14 +380,37 @@ torch::Tensor GemmGroupedV3GatherRS::forward_gather_rs(
     torch::Tensor input, torch::Tensor weight, torch::Tensor splits_cpu, torch::Tensor routing_idx,
     std::optional<torch::Tensor> /*n_tokens_per_rank*/, std::optional<torch::Tensor> input_scale,
     std::optional<torch::Tensor> weight_scale, std::optional<torch::Tensor> output_vec_scale,
-    bool /*fast_accum*/, int64_t /*sm_margin*/, bool with_stream_sync) {
+    bool /*fast_accum*/, int64_t sm_margin, bool with_stream_sync) {
   auto wrap = [](std::optional<torch::Tensor> &t) {
     std::optional<std::vector<torch::Tensor>> v;
     if (t.has_value()) v = std::vector<torch::Tensor>{*t};
     return v;
   };
   return forward_impl({input}, {weight}, splits_cpu, routing_idx, wrap(input_scale), wrap(weight_scale),
-                      wrap(output_vec_scale), with_stream_sync);
+                      wrap(output_vec_scale), with_stream_sync, sm_margin);
+}
+
+torch::Tensor GemmGroupedV3GatherRS::profiling(
+    torch::Tensor input, torch::Tensor weight, torch::Tensor splits_cpu, torch::Tensor routing_idx,
+    std::optional<torch::Tensor> n_tokens_per_rank, std::optional<torch::Tensor> input_scale,
+    std::optional<torch::Tensor> weight_scale, std::optional<torch::Tensor> output_vec_scale, bool fast_accum,
+    int64_t sm_margin, bool with_stream_sync, std::shared_ptr<ProfilingContext> prof_ctx) {
+  ProfilingContext tmp_ctx("__tmp__");
+  ProfilingContext *ctx = prof_ctx ? prof_ctx.get() : &tmp_ctx;
+  auto run = [&]() {
+    return forward_gather_rs(input, weight, splits_cpu, routing_idx, n_tokens_per_rank, input_scale, weight_scale,
+                             output_vec_scale, fast_accum, sm_margin, with_stream_sync);
+  };
+  run();  // argument checks before anything is timed
+  GemmShapeKey key;
+  key.dtype = to_fluxmi_dtype(weight.scalar_type());
+  key.nexperts = static_cast<int32_t>(num_experts_);
+  key.n = static_cast<int32_t>(n_dim_);
+  key.k = static_cast<int32_t>(input.size(1));
+  key.max_rows = static_cast<int32_t>(input.size(0));
+  key.ngroups = 1;
+  if (key.max_rows > 0) profile_schedules(key, ctx, run);
+  return run();  // with the schedule just registered
 }
 
 torch::Tensor GemmGroupedV3GatherRS::forward_gather_rs_multiple(
@@ -295,10 +418,10 @@ torch::Tensor GemmGroupedV3GatherRS::forward_gather_rs_multiple(
     torch::Tensor routing_idx, std::optional<torch::Tensor> /*n_tokens_per_rank*/,
     std::optional<std::vector<torch::Tensor>> input_scale,
     std::optional<std::vector<torch::Tensor>> weight_scale,
-    std::optional<std::vector<torch::Tensor>> output_vec_scale, bool /*fast_accum*/, int64_t /*sm_margin*/,
+    std::optional<std::vector<torch::Tensor>> output_vec_scale, bool /*fast_accum*/, int64_t sm_margin,
     bool with_stream_sync) {
   return forward_impl(inputs, weights, splits_cpu, routing_idx, input_scale, weight_scale, output_vec_scale,
-                      with_stream_sync);
+                      with_stream_sync, sm_margin);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -323,7 +446,7 @@ torch::Tensor GemmGroupedV3::forward(torch::Tensor input, torch::Tensor splits_c
   torch::Tensor out = torch::empty({input.size(0), weight_.size(1)}, input.options().dtype(at::kBFloat16));
   if (input.size(0) == 0) return out;
   torch::Tensor splits_dev = splits_cpu.to(at::kInt).to(input.device(), /*non_blocking=*/true);
-  run_grouped_gemm(input, weight_, splits_dev, out, nullptr, input.size(0), nullptr, nullptr, nullptr, nullptr);
+  run_grouped_gemm(input, weight_, splits_dev, out, nullptr, input.size(0), nullptr, nullptr, nullptr, nullptr, 0);
   return out;
 }
 

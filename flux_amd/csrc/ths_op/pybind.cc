@@ -50,6 +50,20 @@ PYBIND11_MODULE(flux_ths_pybind, m) {
            py::arg("tp_group") = py::none(), py::arg("nnodes") = 1, py::arg("ep_group") = py::none())
       .def("__repr__", &DistEnvTPWithEP::to_string);
 
+  // src/pybind/ths_op.cc:78-92 (ProfilingContext, TuningRecord)
+  py::class_<ProfilingContext, std::shared_ptr<ProfilingContext>>(m, "ProfilingContext")
+      .def(py::init<std::string>(), py::arg("name"))
+      .def("get_code", &ProfilingContext::get_code)
+      .def("get_all_prof_results", &ProfilingContext::get_all_prof_results)
+      .def("get_latest_prof_result", &ProfilingContext::get_latest_prof_result)
+      .def("get_latest_record", &ProfilingContext::get_latest_record)
+      .def("get_all_records", &ProfilingContext::get_all_records);
+  py::class_<TuningRecord>(m, "TuningRecord")
+      .def("__repr__", &TuningRecord::to_string)
+      .def_property_readonly("shape", [](const TuningRecord &r) { return r.key.to_string(); })
+      .def_property_readonly("raster_rows", [](const TuningRecord &r) { return r.best.raster_rows; })
+      .def_property_readonly("sched_flags", [](const TuningRecord &r) { return r.best.sched_flags; });
+
   py::class_<GemmGroupedV3AGScatter>(m, "GemmGroupedV3AGScatter")
       .def(py::init<DistEnvTPWithEP, MoeArguments>(), py::arg("tp_env"), py::arg("moe_args"))
       .def("clear_buffers", &GemmGroupedV3AGScatter::clear_buffers)
@@ -60,7 +74,11 @@ PYBIND11_MODULE(flux_ths_pybind, m) {
       .def("forward_multiple_weights", &GemmGroupedV3AGScatter::forward_multiple_weights, py::arg("inputs_shard"),
            py::arg("weights"), py::arg("splits_gpu"), py::arg("scatter_index"), py::arg("output_scale") = py::none(),
            py::arg("outputs_buf") = py::none(), py::arg("allgather_output") = py::none(),
-           py::arg("fast_accum") = false, py::arg("sm_margin") = 0);
+           py::arg("fast_accum") = false, py::arg("sm_margin") = 0)
+      .def("profiling", &GemmGroupedV3AGScatter::profiling, py::arg("inputs_shard"), py::arg("weights"),
+           py::arg("splits_gpu"), py::arg("scatter_index"), py::arg("output_scale") = py::none(),
+           py::arg("outputs_buf") = py::none(), py::arg("allgather_output") = py::none(),
+           py::arg("fast_accum") = false, py::arg("sm_margin") = 0, py::arg("prof_ctx") = nullptr);
 
   py::class_<GemmGroupedV3GatherRS>(m, "GemmGroupedV3GatherRS")
       .def(py::init<int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, bool>(),
@@ -82,7 +100,12 @@ PYBIND11_MODULE(flux_ths_pybind, m) {
            py::arg("input_scale") = py::none(), py::arg("weight_scale") = py::none(),
            py::arg("output_vec_scale") = py::none(), py::arg("fast_accum") = true, py::arg("sm_margin") = 0,
            py::arg("with_stream_sync") = false)
-      .def("ep_zero_buffer", &GemmGroupedV3GatherRS::ep_zero_buffer);
+      .def("ep_zero_buffer", &GemmGroupedV3GatherRS::ep_zero_buffer)
+      .def("profiling", &GemmGroupedV3GatherRS::profiling, py::arg("input"), py::arg("weight"), py::arg("splits_cpu"),
+           py::arg("routing_idx"), py::arg("n_tokens_per_rank") = py::none(), py::arg("input_scale") = py::none(),
+           py::arg("weight_scale") = py::none(), py::arg("output_vec_scale") = py::none(),
+           py::arg("fast_accum") = false, py::arg("sm_margin") = 0, py::arg("with_stream_sync") = false,
+           py::arg("prof_ctx") = nullptr);
 
   py::class_<GemmGroupedV3>(m, "GemmGroupedV3")
       .def(py::init<torch::Tensor, int64_t>(), py::arg("weight"), py::arg("num_experts"))
@@ -128,6 +151,12 @@ PYBIND11_MODULE(flux_ths_pybind, m) {
     return true;
   });
   // The reference's tuning records select among its generated kernel variants (src/ths_op/ths_op.cc:213-216);
-  // this build has one kernel per element type, so there is nothing to register.
-  m.def("load_tuning_record", [](py::object) {}, py::arg("record"));
+  // here a record selects the tile schedule of the persistent grouped GEMM for one problem shape.
+  m.def("load_tuning_record", [](const TuningRecord &r) { TuningTable::instance().add(r.key, r.best); },
+        py::arg("record"));
+  // Text written by ProfilingContext.get_code(); also read once per process from $FLUX_AMD_TUNING_FILE.
+  m.def("load_tuning_text", [](const std::string &text) { return TuningTable::instance().load_text(text); },
+        py::arg("text"));
+  m.def("clear_tuning_records", []() { TuningTable::instance().clear(); });
+  m.def("num_tuning_records", []() { return TuningTable::instance().size(); });
 }

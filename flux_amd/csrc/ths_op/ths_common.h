@@ -11,6 +11,7 @@
 #include <vector>
 
 #include "fluxmi.h"
+#include "tuning.h"
 
 namespace flux_amd {
 
@@ -66,6 +67,10 @@ struct DistEnvTPWithEP {  // include/flux/ths_op/ths_op.h:117-130; only world si
 // Filled grouped-GEMM argument block (everything on the current stream).
 void run_grouped_gemm(const torch::Tensor &a, const torch::Tensor &b, const torch::Tensor &splits_dev,
                       torch::Tensor &d, const int32_t *gather_a, int64_t max_rows, const float *alpha,
-                      const float *row_scale, const float *col_scale, const float *scalar_dev);
+                      const float *row_scale, const float *col_scale, const float *scalar_dev, int64_t sm_margin);
+
+// Launch tuning of a grouped GEMM: CUs to leave free (Flux's sm_margin) and the tile schedule registered
+// for the problem's shape, if any.
+void apply_launch_tuning(fluxmi_grouped_gemm_args &args, int32_t ngroups, int64_t sm_margin);
 
 }  // namespace flux_amd

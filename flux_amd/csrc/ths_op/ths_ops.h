@@ -17,6 +17,12 @@ class GemmGroupedV3AGScatter {
       torch::Tensor scatter_index, std::optional<std::vector<torch::Tensor>> output_scale,
       std::optional<std::vector<torch::Tensor>> outputs_buf, std::optional<torch::Tensor> allgather_output,
       bool fast_accum, int64_t sm_margin);
+  // forward() under every tile schedule, timed; the fastest is registered for the shape and recorded in
+  // prof_ctx (gemm_grouped_v3_ag_scatter.cc:520-612).
+  torch::Tensor profiling(torch::Tensor inputs_shard, torch::Tensor weights, torch::Tensor splits_gpu,
+                          torch::Tensor scatter_index, std::optional<torch::Tensor> output_scale,
+                          std::optional<torch::Tensor> outputs_buf, std::optional<torch::Tensor> allgather_output,
+                          bool fast_accum, int64_t sm_margin, std::shared_ptr<ProfilingContext> prof_ctx);
 
  private:
   std::vector<torch::Tensor> forward_impl(torch::Tensor inputs_shard, std::vector<torch::Tensor> weights,
@@ -49,13 +55,21 @@ class GemmGroupedV3GatherRS {
                                            std::optional<std::vector<torch::Tensor>> output_vec_scale,
                                            bool fast_accum, int64_t sm_margin, bool with_stream_sync);
   void ep_zero_buffer() {}  // expert-parallel scratch does not exist at world size 1
+  // forward_gather_rs() under every tile schedule, timed; the fastest is registered for the shape and
+  // recorded in prof_ctx (gemm_grouped_v3_gather_rs.cc:903-1000).
+  torch::Tensor profiling(torch::Tensor input, torch::Tensor weight, torch::Tensor splits_cpu,
+                          torch::Tensor routing_idx, std::optional<torch::Tensor> n_tokens_per_rank,
+                          std::optional<torch::Tensor> input_scale, std::optional<torch::Tensor> weight_scale,
+                          std::optional<torch::Tensor> output_vec_scale, bool fast_accum, int64_t sm_margin,
+                          bool with_stream_sync, std::shared_ptr<ProfilingContext> prof_ctx);
 
  private:
   torch::Tensor forward_impl(std::vector<torch::Tensor> inputs, std::vector<torch::Tensor> weights,
                              torch::Tensor splits_cpu, torch::Tensor routing_idx,
                              std::optional<std::vector<torch::Tensor>> input_scale,
                              std::optional<std::vector<torch::Tensor>> weight_scale,
-                             std::optional<std::vector<torch::Tensor>> output_vec_scale, bool with_stream_sync);
+                             std::optional<std::vector<torch::Tensor>> output_vec_scale, bool with_stream_sync,
+                             int64_t sm_margin);
   void lazy_init(const torch::Tensor &like);
   int64_t num_experts_, max_m_, n_dim_, topk_, max_input_groups_;
   bool inter_fp32_ = true;

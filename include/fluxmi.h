@@ -106,7 +106,15 @@ typedef struct fluxmi_grouped_gemm_args {
   float scalar_scale;       /* host scalar, 1.0f for none (Flux `input_scale[0]` is passed by pointer below) */
   int32_t d_fp32;           /* 0: D is bf16; 1: D is fp32 [max_rows, N] (unrounded layer1 intermediate) */
   const float *scalar_scale_dev; /* device [1] or NULL; multiplied in if given */
+  /* Launch tuning; all zero = defaults.  None of them changes a result bit. */
+  int32_t cu_margin;     /* compute units left free for other work (Flux `sm_margin`) */
+  int32_t raster_rows;   /* row tiles of an expert walked together over all weight panels; 0 = 8 */
+  int32_t sched_flags;   /* FLUXMI_SCHED_* */
+  int32_t reserved;      /* must be 0 */
 } fluxmi_grouped_gemm_args;
+
+#define FLUXMI_SCHED_WHOLE_TAIL_TILES 1 /* do not cut the tiles of the last, partly filled round into pieces */
+#define FLUXMI_SCHED_NO_HALF_TILES 2    /* run the last row tile of an expert 256 rows high even if 128 cover it */
 
 size_t fluxmi_grouped_gemm_workspace_bytes(const fluxmi_grouped_gemm_args *args);
 int fluxmi_grouped_gemm(const fluxmi_grouped_gemm_args *args, void *workspace,

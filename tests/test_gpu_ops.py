@@ -192,3 +192,77 @@ def test_fp8_layer1_through_ops():
     ref = layers.topk_gather_reduce_fp32(z, wl.scatter_index.reshape(-1), k)
     err = float((out.float().cpu() - ref).norm() / ref.norm())
     assert err < 3e-2, err
+
+
+def test_profiling_registers_a_schedule_and_keeps_results(c1):
+    """profiling() of both layer ops: every tile schedule gives the bits of forward(); the fastest is recorded in
+    the context, registered for the shape, and its text form loads back."""
+    wl = c1
+    m = flux_amd.flux_ths_pybind
+    m.clear_tuning_records()
+    t, k, e, h, f = wl.tokens, wl.topk, wl.experts, wl.hidden, wl.ffn
+    x, w1, w2 = (wl.tensors[n].cuda() for n in ("x", "w1", "w2"))
+    splits_gpu = torch.from_numpy(wl.splits).cuda()
+    scatter_index = torch.from_numpy(wl.scatter_index).cuda()
+    op0 = flux_amd.GemmGroupedV3AGScatter(flux_amd.DistEnvTPWithEP(None, 1, None),
+                                          flux_amd.MoeArguments(t, h, f, e, k, torch.bfloat16))
+    ref0 = op0.forward(x, w1, splits_gpu, scatter_index)
+    ctx = flux_amd.ProfilingContext("c1")
+    out0 = op0.profiling(x, w1, splits_gpu, scatter_index, prof_ctx=ctx)
+    assert torch.equal(out0, ref0)
+    assert m.num_tuning_records() == 1
+    rec = ctx.get_latest_record()
+    assert f"experts={e} n={f} k={h} rows={t * k} groups=1" in rec.shape
+    assert rec.raster_rows in (4, 8, 16) and 0 <= rec.sched_flags <= 3
+    assert ctx.get_latest_prof_result().count("TopK=") == 5
+    assert torch.equal(op0.forward(x, w1, splits_gpu, scatter_index), ref0)  # now under the registered schedule
+
+    op1 = flux_amd.GemmGroupedV3GatherRS(e, t * k, h, k, 0, 1, 1, 1)
+    routing_idx = scatter_index.view(-1)
+    ref1 = op1.forward_gather_rs(ref0, w2, torch.from_numpy(wl.splits), routing_idx)
+    out1 = op1.profiling(ref0, w2, torch.from_numpy(wl.splits), routing_idx, prof_ctx=ctx)
+    assert torch.equal(out1, ref1)
+    assert m.num_tuning_records() == 2 and len(ctx.get_all_records()) == 2 and len(ctx.get_all_prof_results()) == 2
+    code = ctx.get_code()
+    assert code.count("fluxmi_gemm_tuning") == 2
+    m.clear_tuning_records()
+    assert m.load_tuning_text(code) == 2
+    m.clear_tuning_records()
+    m.load_tuning_record(rec)
+    assert m.num_tuning_records() == 1
+    m.clear_tuning_records()
+    # without a context the profiler still runs and registers
+    op0.profiling(x, w1, splits_gpu, scatter_index)
+    assert m.num_tuning_records() == 1
+    m.clear_tuning_records()
+
+
+@pytest.mark.parametrize("raster_rows,flags,margin", [(4, 0, 0), (16, 1, 0), (8, 2, 0), (1, 3, 0), (8, 0, 40), (8, 0, 255),
+                                                       (8, 0, 1000)])
+def test_tile_schedules_and_cu_margin_do_not_change_a_bit(raster_rows, flags, margin):
+    """Launch tuning (raster group height, whole tail tiles, no half tiles) and sm_margin move tiles between
+    workgroups; every output bit must stay what the default schedule gives."""
+    from flux_amd import capi
+    rng = np.random.default_rng(5)
+    g = torch.Generator().manual_seed(5)
+    experts, rows, n, kk = 6, 5000, 768, 512
+    cnt = rng.multinomial(rows, [0.4, 0.02, 0.0, 0.28, 0.2, 0.1]).astype(np.int32)
+    a = torch.randn(rows, kk, generator=g).to(torch.bfloat16).cuda()
+    w = (torch.randn(experts, n, kk, generator=g) * 0.05).to(torch.bfloat16).cuda()
+    sp = torch.from_numpy(cnt).cuda()
+    base = capi.grouped_gemm(a, w, sp)
+    close(base, layers.grouped_gemm_fp32(a.cpu(), w.cpu(), cnt))
+    got = capi.grouped_gemm(a, w, sp, cu_margin=margin, raster_rows=raster_rows, sched_flags=flags)
+    assert torch.equal(got, base)
+
+
+def test_sm_margin_through_the_ops(c1):
+    wl = c1
+    t, k, e, h, f = wl.tokens, wl.topk, wl.experts, wl.hidden, wl.ffn
+    x, w1 = wl.tensors["x"].cuda(), wl.tensors["w1"].cuda()
+    op0 = flux_amd.GemmGroupedV3AGScatter(flux_amd.DistEnvTPWithEP(None, 1, None),
+                                          flux_amd.MoeArguments(t, h, f, e, k, torch.bfloat16))
+    sp, si = torch.from_numpy(wl.splits).cuda(), torch.from_numpy(wl.scatter_index).cuda()
+    assert torch.equal(op0.forward(x, w1, sp, si, sm_margin=28), op0.forward(x, w1, sp, si))
+    with pytest.raises(RuntimeError, match="sm_margin"):
+        op0.forward(x, w1, sp, si, sm_margin=-1)

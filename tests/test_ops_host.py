@@ -12,12 +12,14 @@ def test_module_exports_reference_names():
     m = flux_amd.flux_ths_pybind
     for name in ("MoeArguments", "DistEnvTPWithEP", "GemmGroupedV3AGScatter", "GemmGroupedV3GatherRS", "GemmGroupedV3",
                  "Quantization", "calc_scatter_index", "topk_scatter_reduce", "bitwise_check", "init_flux_shm",
-                 "uniform_initialize", "load_tuning_record"):
+                 "uniform_initialize", "load_tuning_record", "ProfilingContext", "TuningRecord"):
         assert hasattr(m, name), name
         assert getattr(flux_amd, name) is getattr(m, name)
-    for cls, methods in ((m.GemmGroupedV3AGScatter, ("forward", "forward_multiple_weights", "clear_buffers")),
+    for cls, methods in ((m.GemmGroupedV3AGScatter, ("forward", "forward_multiple_weights", "clear_buffers", "profiling")),
                          (m.GemmGroupedV3GatherRS, ("forward_gather_rs", "forward_gather_rs_multiple",
-                                                    "forward_gather_rs_no_zerobuffer", "ep_zero_buffer")),
+                                                    "forward_gather_rs_no_zerobuffer", "ep_zero_buffer", "profiling")),
+                         (m.ProfilingContext, ("get_code", "get_all_prof_results", "get_latest_prof_result",
+                                               "get_latest_record", "get_all_records")),
                          (m.Quantization, ("quantize_vector_blockwise", "quantize_square_blockwise",
                                            "batch_quantize_square_blockwise"))):
         for meth in methods:
@@ -61,7 +63,8 @@ def test_world_size_above_one_is_rejected():
     with pytest.raises(RuntimeError, match="nnodes"):
         flux_amd.DistEnvTPWithEP(None, 2)
     flux_amd.init_flux_shm(None)
-    flux_amd.load_tuning_record(object())
+    with pytest.raises(TypeError):
+        flux_amd.load_tuning_record(object())  # takes a TuningRecord (from a ProfilingContext)
     with pytest.raises(RuntimeError, match="unsupported dtype"):
         flux_amd.uniform_initialize(torch.zeros(4), 1, 0.0, 1.0)
 
@@ -97,3 +100,29 @@ def test_dtype_and_device_checks():
     assert flux_amd.bitwise_check(torch.arange(6).view(2, 3), torch.arange(6).view(2, 3))
     assert not flux_amd.bitwise_check(torch.zeros(3), torch.zeros(4))
     assert not flux_amd.bitwise_check(torch.tensor([0.0]), torch.tensor([-0.0]))
+
+
+def test_tuning_text_round_trip_and_errors():
+    """The shape-keyed schedule table: text in, records counted, malformed lines rejected with their line number."""
+    m = flux_amd.flux_ths_pybind
+    m.clear_tuning_records()
+    text = ("# comment\n"
+            "fluxmi_gemm_tuning dtype=bf16 experts=8 n=14336 k=4096 rows=16384 groups=1 raster_rows=16 sched_flags=1\n"
+            "\n"
+            "fluxmi_gemm_tuning dtype=e4m3 experts=32 n=7168 k=2048 rows=32768 groups=1 raster_rows=4 sched_flags=0  # x\n")
+    assert m.load_tuning_text(text) == 2
+    assert m.num_tuning_records() == 2
+    assert m.load_tuning_text(text) == 2 and m.num_tuning_records() == 2   # same keys: replaced, not duplicated
+    for bad, what in (("fluxmi_gemm_tuning dtype=bf16 experts=8", "missing fields"),
+                      ("something else", "expected 'fluxmi_gemm_tuning'"),
+                      ("fluxmi_gemm_tuning dtype=fp64 experts=1 n=1 k=1 rows=1 groups=1 raster_rows=1 sched_flags=0", "unknown dtype"),
+                      ("fluxmi_gemm_tuning dtype=bf16 experts=x n=1 k=1 rows=1 groups=1 raster_rows=1 sched_flags=0", "bad number"),
+                      ("fluxmi_gemm_tuning dtype=bf16 experts=1 n=1 k=1 rows=1 groups=1 raster_rows=1 sched_flags=64", "out of range")):
+        with pytest.raises(RuntimeError, match=what):
+            m.load_tuning_text("# first line\n" + bad)
+    m.clear_tuning_records()
+    assert m.num_tuning_records() == 0
+    ctx = m.ProfilingContext("empty")
+    assert "empty" in ctx.get_code() and ctx.get_all_records() == []
+    with pytest.raises(RuntimeError, match="no latest prof results"):
+        ctx.get_latest_record()
