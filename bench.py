@@ -174,17 +174,18 @@ def main():
         b_gr = m * h * 2 + m * 4 + m * 4 + t * h * 2
         kernels["gather_reduce_bf16_weighted"] = {"ms": round(t_gr, 4), "gbs": round(b_gr / t_gr * 1e-6, 1),
                                                   "frac_hbm": round(b_gr / t_gr * 1e-6 / PEAK_HBM_GBS, 4)}
-        # The reduce at the C4 and C5 shapes (top-6 of 16384 tokens x 2048, top-8 of 4096 tokens x 7168), bf16 rows
-        # with per-row weights, routing = a random permutation of the rows.
-        for tag, (t2, k2, n2) in (("c4", (16384, 6, 2048)), ("c5", (4096, 8, 7168))):
-            m2 = t2 * k2
+        # The reduce at the C4 and C5 shapes (top-6 of 16384 tokens x 2048, top-8 of 4096 tokens x 7168) with those
+        # workloads' own routing (stable scatter index, per-row top-k weights), bf16 rows.
+        for tag in ("C4", "C5"):
+            wl2, _ = configs.make_routing(tag)
+            t2, k2, n2, m2 = wl2.tokens, wl2.topk, wl2.hidden, wl2.rows
             z2 = torch.randn(m2, n2, generator=gen, device=dev).to(torch.bfloat16)
-            idx2 = torch.randperm(m2, generator=gen, device=dev).to(torch.int32)
-            w2r = torch.rand(m2, generator=gen, device=dev)
+            idx2 = torch.from_numpy(wl2.scatter_index.reshape(-1)).to(dev)
+            w2r = wl2.row_weight.to(dev)
             o2 = torch.empty(t2, n2, dtype=torch.bfloat16, device=dev)
             t_g2 = time_loop(torch, lambda: capi.topk_gather_reduce(z2, idx2, k2, w2r, out=o2), 30)
             b_g2 = m2 * n2 * 2 + m2 * 8 + t2 * n2 * 2
-            kernels[f"gather_reduce_bf16_weighted_{tag}_shape"] = {
+            kernels[f"gather_reduce_bf16_weighted_{tag.lower()}"] = {
                 "ms": round(t_g2, 4), "gbs": round(b_g2 / t_g2 * 1e-6, 1),
                 "frac_hbm": round(b_g2 / t_g2 * 1e-6 / PEAK_HBM_GBS, 4)}
             del z2, idx2, w2r, o2
