@@ -4,11 +4,15 @@
 // columns, k-step of 64 bytes per row (32 bf16 or 64 fp8).  Both operand tiles are staged in LDS by
 // direct-to-LDS global loads (no register staging) in a ring of five 32 KiB stages; the row gather of A
 // is folded into the per-lane global address of those loads.  Each wave owns a 128 x 128 quarter of the
-// macro tile (4x4 MFMA blocks of 32x32, 256 fp32 accumulator registers) and runs a software pipeline
-// of its own: while the MFMAs of k-step s run on one set of fragment registers, the fragments of step
-// s+1 are read from LDS into a second set and the ring fills of steps s+4 / s+5 are issued, all in a
-// fixed interleaving (one fragment read per MFMA over the first half of the step, one fill every
-// fourth MFMA).  One workgroup barrier per k-step publishes the landed stage.
+// macro tile (bf16: 8x8 MFMA blocks of 16x16, fp8: 4x4 blocks of 32x32; 256 fp32 accumulator registers
+// either way) and runs a software pipeline of its own: while the MFMAs of k-step s run on one set of
+// fragment registers, the fragments of step s+1 are read from LDS into a second set and the ring fills of
+// steps s+4 / s+5 are issued, all in a fixed interleaving (the 16 fragment reads spread evenly over the
+// first half of the step's MFMAs, the 8 fills evenly over the whole step).  One workgroup barrier per
+// k-step publishes the landed stage.
+//
+// A launch may carry up to four weight tensors ("groups") that multiply the same rows, each with its own
+// output: their column tiles are numbered through one schedule (GemmParams::ngroups).
 //
 // Ring fills are issued in pairs of k-steps: the two 64-byte halves of a 128-byte line are requested
 // back to back (they go to different stages), so the second request hits the line the first one
