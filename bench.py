@@ -211,6 +211,15 @@ def main():
         kernels["gemm_fp8_c5_layer1"] = {"ms": round(t_f8, 4), "tflops": round(f_f8 / t_f8 * 1e-9, 1),
                                          "frac_fp8_peak": round(f_f8 / t_f8 * 1e-9 / PEAK_FP8_TFLOPS, 4)}
         del a8, b8, d5
+        # ... and layer0 of the same share: K = 7168, N = 2048 (per-row and per-column scales, no top-k weight)
+        a8 = torch.randn(m5, n5, generator=gen, device=dev).to(torch.float8_e4m3fn)
+        b8 = (torch.randn(e5, k5, n5, generator=gen, device=dev)).to(torch.float8_e4m3fn)
+        cs0 = torch.rand(e5, k5, generator=gen, device=dev)
+        d5 = torch.empty(m5, k5, dtype=torch.bfloat16, device=dev)
+        t_f8 = time_loop(torch, lambda: capi.grouped_gemm(a8, b8, sp5, out=d5, row_scale=rs5, col_scale=cs0), 20)
+        kernels["gemm_fp8_c5_layer0"] = {"ms": round(t_f8, 4), "tflops": round(f_f8 / t_f8 * 1e-9, 1),
+                                         "frac_fp8_peak": round(f_f8 / t_f8 * 1e-9 / PEAK_FP8_TFLOPS, 4)}
+        del a8, b8, d5, cs0
         # The same two C3 GEMMs as a loop of library GEMMs (torch.mm = hipBLASLt), one per expert, on rows that
         # are already gathered and contiguous: the path a port without a grouped kernel would take.  Reported
         # beside the grouped kernel for comparison; not part of the step.
