@@ -481,18 +481,24 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
         constexpr int r = decltype(R)::value;
         if constexpr (r * RSPAN / NR == t) read_one(std::integral_constant<int, (u + 1) % STG>{}, R, xn, wn_);
       });
+      // Loads of this slot first, M0 writes for the loads of the next slot after them: a whole fill placed
+      // here (fill_one writes M0 itself) must not come between another fill's M0 write and its load.
       static_for<0, 2 * LOADS>([&](auto D) {
         constexpr int d = decltype(D)::value;
         constexpr int at = (d * (2 * NM) / (2 * LOADS) + 1) % (2 * NM);
-        if constexpr (at % NM != 0) {  // the slot before is in the same step
-          if constexpr (at - 1 == t + (even ? 0 : NM))
-            fill_m0(std::integral_constant<int, (e0 + LA + (d & 1)) % STG>{}, std::integral_constant<int, (d >> 1)>{});
-          if constexpr (at == t + (even ? 0 : NM))
+        if constexpr (at == t + (even ? 0 : NM)) {
+          if constexpr (at % NM != 0)  // the slot before is in the same step: M0 was written there
             fill_go(std::integral_constant<int, (d >> 1)>{}, kbase + (e0 + LA + (d & 1)) * KBYTES);
-        } else if constexpr (at == t + (even ? 0 : NM)) {
-          fill_one(std::integral_constant<int, (e0 + LA + (d & 1)) % STG>{}, std::integral_constant<int, (d >> 1)>{},
-                   kbase + (e0 + LA + (d & 1)) * KBYTES);
+          else
+            fill_one(std::integral_constant<int, (e0 + LA + (d & 1)) % STG>{}, std::integral_constant<int, (d >> 1)>{},
+                     kbase + (e0 + LA + (d & 1)) * KBYTES);
         }
+      });
+      static_for<0, 2 * LOADS>([&](auto D) {
+        constexpr int d = decltype(D)::value;
+        constexpr int at = (d * (2 * NM) / (2 * LOADS) + 1) % (2 * NM);
+        if constexpr (at % NM != 0 && at - 1 == t + (even ? 0 : NM))
+          fill_m0(std::integral_constant<int, (e0 + LA + (d & 1)) % STG>{}, std::integral_constant<int, (d >> 1)>{});
       });
       mfma_slot<ELT, MBK, NBK>(t, xc, wc, acc);
       __builtin_amdgcn_sched_barrier(0);
@@ -729,8 +735,11 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
     const int gcol = g * tiles_n1 * BN;  // first virtual column of the weight group
     t.n0 = (nt - g * tiles_n1) * BN;
     if (item < full_items || pieces == 1) {
-      // The last row tile of an expert is run 128 rows high when that covers its rows.
-      t.kind = (rows_e - t.m0 > 128 || !half_tiles) ? 0 : 1;
+      // The last row tile of an expert is run 128 rows high when that covers its rows, the last column
+      // tile 128 columns wide when that covers its columns (N = 1408: the sixth tile holds 128 columns).
+      const bool low = half_tiles && rows_e - t.m0 <= 128;
+      const bool narrow = half_tiles && p.n - t.n0 <= 128;
+      t.kind = low ? (narrow ? 3 : 1) : (narrow ? 2 : 0);
     } else if (pieces == 2) {
       t.n0 += piece * 128;
       t.kind = t.n0 < p.n ? 2 : -1;

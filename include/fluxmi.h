@@ -114,7 +114,7 @@ typedef struct fluxmi_grouped_gemm_args {
 } fluxmi_grouped_gemm_args;
 
 #define FLUXMI_SCHED_WHOLE_TAIL_TILES 1 /* do not cut the tiles of the last, partly filled round into pieces */
-#define FLUXMI_SCHED_NO_HALF_TILES 2    /* run the last row tile of an expert 256 rows high even if 128 cover it */
+#define FLUXMI_SCHED_NO_HALF_TILES 2    /* run the last row tile of an expert 256 rows high even if 128 cover it, and the last column tile 256 wide even if 128 cover it */
 
 size_t fluxmi_grouped_gemm_workspace_bytes(const fluxmi_grouped_gemm_args *args);
 int fluxmi_grouped_gemm(const fluxmi_grouped_gemm_args *args, void *workspace,

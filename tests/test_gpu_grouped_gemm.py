@@ -234,7 +234,11 @@ def quantise(t_bf16):
 
 
 @pytest.mark.parametrize("experts,rows,n,k,seed", [(1, 256, 256, 64, 0), (4, 1000, 512, 256, 1), (8, 2000, 1024, 1024, 2),
-                                                   (3, 300, 264, 2048, 3), (2, 40, 8, 100, 4), (3, 700, 264, 192, 5), (2, 300, 512, 960, 6), (4, 1100, 384, 1536, 7)])
+                                                   (3, 300, 264, 2048, 3), (2, 40, 8, 100, 4), (3, 700, 264, 192, 5), (2, 300, 512, 960, 6), (4, 1100, 384, 1536, 7),
+                                                   # 128x128 and 256x128 tiles (last rows of an expert, last columns of N) over
+                                                   # 18 and more k-steps: the unrolled trips of the narrow tile shapes
+                                                   (1, 100, 128, 2048, 8), (1, 100, 384, 1536, 9), (1, 256, 128, 1152, 10),
+                                                   (2, 600, 640, 1280, 11)])
 def test_fp8_against_dequant_matmul(experts, rows, n, k, seed):
     from flux_amd import capi
     print(f"[case] grouped_gemm fp8 E={experts} rows={rows} N={n} K={k}", flush=True)
