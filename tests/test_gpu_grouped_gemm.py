@@ -311,3 +311,30 @@ def test_fp8_multiple_weight_groups_one_launch():
         ref = layers.grouped_gemm_fp32(a8.float(), ws[i].float(), split, row_scale=rs)
         err = (outs[i].float().cpu() - ref).norm() / ref.norm()
         assert float(err) < FP8_FROB
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp8"])
+@pytest.mark.parametrize("row_tiles,what", [(17, "16 tiles past a full round: cut into 128x128 pieces"),
+                                            (21, "80 tiles past a full round: cut into 256x128 pieces")])
+def test_last_round_cut_into_pieces(dtype, row_tiles, what):
+    """More tiles than CUs with a short last round (256 CUs, 16 column tiles): the schedule cuts the tiles of
+    that round into pieces, which run the narrow tile shapes at every piece offset, here over 20 k-steps."""
+    from flux_amd import capi
+    print(f"[case] grouped_gemm {dtype} tail pieces, {row_tiles} row tiles x 16 column tiles: {what}", flush=True)
+    g = torch.Generator().manual_seed(row_tiles)
+    rows, n = 256 * row_tiles, 4096
+    k = 640 if dtype == "bf16" else 1280          # 20 k-steps of 64 bytes
+    split = np.array([rows - 700, 700], dtype=np.int32)
+    if dtype == "bf16":
+        a = torch.randn(rows, k, generator=g).to(torch.bfloat16)
+        w = (torch.randn(2, n, k, generator=g) * 0.05).to(torch.bfloat16)
+    else:
+        a = torch.randn(rows, k, generator=g).to(torch.float8_e4m3fn)
+        w = torch.randn(2, n, k, generator=g).to(torch.float8_e4m3fn)
+    ref = layers.grouped_gemm_fp32(a.float(), w.float(), split)
+    out = capi.grouped_gemm(a.cuda(), w.cuda(), torch.from_numpy(split).cuda()).float().cpu()
+    if dtype == "bf16":
+        assert_close(out, ref, what)
+    else:
+        assert float((out - ref).norm() / ref.norm()) < FP8_FROB
+        assert torch.allclose(out, ref, rtol=1e-2, atol=1e-2 * float(ref.abs().max()))
