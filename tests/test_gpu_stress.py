@@ -60,3 +60,41 @@ def test_random_ragged_steps(seed):
     got = out.float()
     bad = (got - ref).abs() > 1e-2 + 1e-2 * ref.abs()
     assert not bool(bad.any()), f"{int(bad.sum())} of {bad.numel()} outside tolerance, max {float((got - ref).abs().max())}"
+
+
+@pytest.mark.parametrize("seed", range(10))
+@pytest.mark.parametrize("dtype", ["bf16", "fp8"])
+def test_random_ragged_gemms_all_tile_shapes(dtype, seed):
+    """One grouped GEMM per case over random splits (empty and tiny experts included), N that ends in a narrow
+    column tile or not, K from one k-step to fifty, and enough rows that some cases run more tiles than CUs and
+    cut their last round into pieces; per-row and per-column scales in the epilogue.  Reference: fp32 matmuls of
+    the same values on the GPU."""
+    from flux_amd import capi
+    rng = np.random.default_rng(5000 + seed)
+    experts = int(rng.choice([1, 3, 8, 32]))
+    rows = int(rng.choice([37, 900, 5000, 20000, 40000]))
+    n = int(rng.choice([128, 264, 384, 1024, 2048]))
+    kbytes = int(rng.choice([64, 640, 1280, 2048, 3200]))
+    k = kbytes if dtype == "fp8" else kbytes // 2
+    p = rng.random(experts) ** 3 + 1e-3
+    if experts > 2:
+        p[int(rng.integers(0, experts))] = 0.0
+    split = rng.multinomial(rows, p / p.sum()).astype(np.int32)
+    print(f"[case] stress gemm {dtype} seed={seed} E={experts} rows={rows} N={n} K={k} split[:8]={split[:8]}", flush=True)
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    a = torch.randn(rows, k, generator=g, device="cuda")
+    w = torch.randn(experts, n, k, generator=g, device="cuda") * (1.0 if dtype == "fp8" else k ** -0.5)
+    a = a.to(torch.float8_e4m3fn if dtype == "fp8" else torch.bfloat16)
+    w = w.to(torch.float8_e4m3fn if dtype == "fp8" else torch.bfloat16)
+    rs = torch.rand(rows, generator=g, device="cuda") + 0.5
+    cs = (torch.rand(experts, n, generator=g, device="cuda") + 0.5) * (k ** -0.5 if dtype == "fp8" else 1.0)
+    out = capi.grouped_gemm(a, w, torch.from_numpy(split).cuda(), row_scale=rs, col_scale=cs).float()
+    ref = torch.zeros(rows, n, dtype=torch.float32, device="cuda")
+    off = 0
+    for e, cnt in enumerate(split):
+        cnt = int(cnt)
+        if cnt:
+            ref[off:off + cnt] = (a[off:off + cnt].float() @ w[e].float().t()) * rs[off:off + cnt, None] * cs[e][None, :]
+        off += cnt
+    bad = (out - ref).abs() > 1e-2 + 1e-2 * ref.abs()
+    assert not bool(bad.any()), f"{int(bad.sum())} of {bad.numel()} outside tolerance, max {float((out - ref).abs().max())}"
