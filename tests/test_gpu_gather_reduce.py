@@ -48,6 +48,23 @@ def test_fp32_intermediate_input(tokens, topk, n, groups):
     assert_close(out, ref)
 
 
+@pytest.mark.parametrize("tokens,topk,n,groups,weighted", [(50, 2, 2048, 2, True), (33, 8, 7168, 1, True), (20, 4, 264, 3, False),
+                                                           (3000, 2, 520, 1, True), (7, 6, 4096, 4, True)])
+def test_fp32_input_unrolled_topk_groups_and_dropped_rows(tokens, topk, n, groups, weighted):
+    """fp32 rows with the unrolled top-k instances (two strided 16-byte units per lane): several input groups,
+    rows narrower and wider than a pass, few tokens (rows split over workgroups), dropped rows."""
+    from flux_amd import capi
+    g = torch.Generator().manual_seed(tokens + n)
+    m = tokens * topk
+    inter = [torch.randn(m, n, generator=g) for _ in range(groups)]
+    idx = torch.randperm(m, generator=g).to(torch.int32)
+    idx[::5] = -1
+    w = torch.rand(m, generator=g) if weighted else None
+    ref = layers.topk_gather_reduce_fp32(inter, idx.numpy(), topk, w, scale=0.5)
+    out = capi.topk_gather_reduce([t.cuda() for t in inter], idx.cuda(), topk, None if w is None else w.cuda(), 0.5)
+    assert_close(out, ref)
+
+
 def test_dropped_rows_and_identity():
     from flux_amd import capi
     g = torch.Generator().manual_seed(9)
