@@ -88,7 +88,19 @@ def test_random_ragged_gemms_all_tile_shapes(dtype, seed):
     w = w.to(torch.float8_e4m3fn if dtype == "fp8" else torch.bfloat16)
     rs = torch.rand(rows, generator=g, device="cuda") + 0.5
     cs = (torch.rand(experts, n, generator=g, device="cuda") + 0.5) * (k ** -0.5 if dtype == "fp8" else 1.0)
-    out = capi.grouped_gemm(a, w, torch.from_numpy(split).cuda(), row_scale=rs, col_scale=cs).float()
+    # odd seeds: A is gathered through a permutation and D scattered through another one
+    gather = scatter = None
+    src = a
+    if seed % 2:
+        gather = torch.randperm(rows, generator=g, device="cuda").to(torch.int32)
+        scatter = torch.randperm(rows, generator=g, device="cuda").to(torch.int32)
+        src = torch.empty_like(a)
+        src.view(torch.uint8 if dtype == "fp8" else torch.int16)[gather.long()] = \
+            a.view(torch.uint8 if dtype == "fp8" else torch.int16)          # src[gather[r]] = a[r]
+    out = capi.grouped_gemm(src, w, torch.from_numpy(split).cuda(), row_scale=rs, col_scale=cs, gather_a=gather,
+                            scatter_d=scatter).float()
+    if scatter is not None:
+        out = out[scatter.long()]                                           # back to sorted-row order
     ref = torch.zeros(rows, n, dtype=torch.float32, device="cuda")
     off = 0
     for e, cnt in enumerate(split):
