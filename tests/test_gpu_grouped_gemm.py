@@ -166,6 +166,24 @@ def test_bf16_k_loop_boundaries(k):
     assert torch.allclose(out32.cpu(), ref, rtol=1e-4, atol=1e-3), float((out32.cpu() - ref).abs().max())
 
 
+@pytest.mark.parametrize("k", [192, 320, 832, 896, 960, 1088, 1152, 1216, 1472, 1536, 1600, 1728, 1792, 1856, 2624, 7168])
+def test_fp8_k_loop_boundaries(k):
+    """The same seams for the fp8 kernel (a k-step is 64 elements): every tile shape occurs (full tiles, 128-row
+    tiles, the 8-column last tile as a 256x128 and a 128x128 tile), with K on either side of the hand-over from the
+    unrolled trips to the pair-wise tail of each shape's ring, odd numbers of k-steps, and one long K."""
+    from flux_amd import capi
+    print(f"[case] grouped_gemm fp8 k-loop seams K={k}", flush=True)
+    g = torch.Generator().manual_seed(k)
+    split = np.array([300, 0, 129, 520, 77], dtype=np.int32)
+    rows, n = int(split.sum()), 520
+    a = torch.randn(rows, k, generator=g).to(torch.float8_e4m3fn)
+    w = torch.randn(len(split), n, k, generator=g).to(torch.float8_e4m3fn)
+    ref = layers.grouped_gemm_fp32(a.float(), w.float(), split)
+    out32 = capi.grouped_gemm(a.cuda(), w.cuda(), torch.from_numpy(split).cuda(), out_dtype=torch.float32).cpu()
+    # products of e4m3 values are exact in fp32; only the summation order differs
+    assert torch.allclose(out32, ref, rtol=1e-4, atol=1e-3 * k ** 0.5), float((out32 - ref).abs().max())
+
+
 def sampled_rows(split, per_expert, rng):
     off = routing.offsets(split)
     rows = []
