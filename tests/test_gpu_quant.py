@@ -60,7 +60,8 @@ def test_all_finite_patterns_fixed_scale(scale):
     (16, 256, 0, False, 0.0), (16, 256, 128, True, 0.0), (130, 384, 128, True, 0.0), (5, 200, 128, False, 0.0),
     (3, 8, 0, False, 0.0), (129, 136, 128, True, 0.0), (257, 7168, 0, False, 0.0), (64, 2048, 0, False, 1e-3),
     (33, 1000, 0, False, 0.0), (9, 4104, 0, False, 0.0), (4, 16384, 0, False, 0.0), (3, 20000, 0, False, 0.0),
-    (70, 1536, 128, False, 0.5)])
+    (70, 1536, 128, False, 0.5), (7, 4096, 0, False, 0.0), (6, 3000, 0, False, 0.0), (11, 1024, 128, False, 0.0),
+    (6, 7168, 128, False, 0.0), (2, 640, 128, False, 0.0)])
 def test_shapes_against_oracle(rows, cols, block, permute, eps):
     print(f"[case] quant rows={rows} cols={cols} block={block} permute={permute} eps={eps}", flush=True)
     rng = np.random.default_rng(rows * 131 + cols)
