@@ -111,12 +111,31 @@ def build_ths_op(force=True):
     return out
 
 
+CAPI_SMOKE = os.path.join(LIB_DIR, "capi_smoke")
+
+
+def build_capi_smoke(force=True):
+    """tests/capi_smoke.c: the C-ABI driven from plain C + the HIP runtime (no torch), linked against the library."""
+    src = os.path.join(ROOT, "tests", "capi_smoke.c")
+    if not os.path.exists(src):
+        return None
+    if not force and _newer(CAPI_SMOKE, [src, KERNEL_LIB, os.path.join(INCLUDE, "fluxmi.h")]):
+        return CAPI_SMOKE
+    _run(["gcc", "-O1", "-std=c11", "-ffp-contract=off", "-D__HIP_PLATFORM_AMD__=1", "-I/opt/rocm/include",
+          f"-I{INCLUDE}", src, "-o", CAPI_SMOKE, f"-L{LIB_DIR}", "-lfluxmi_kernels", "-L/opt/rocm/lib", "-lamdhip64",
+          "-lm", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath,/opt/rocm/lib"])
+    return CAPI_SMOKE
+
+
 def build_all(force=True, kernels_only=False):
     libs = [build_kernels(force)]
     if not kernels_only:
         ext = build_ths_op(force)
         if ext:
             libs.append(ext)
+        smoke = build_capi_smoke(force)
+        if smoke:
+            libs.append(smoke)
     return libs
 
 
