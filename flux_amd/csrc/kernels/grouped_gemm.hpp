@@ -82,6 +82,7 @@ struct GemmParams {
   int32_t ngroups;
   int32_t raster_rows;  // row tiles per raster group, >= 1
   int32_t sched_flags;  // FLUXMI_SCHED_*
+  int32_t nt_stores;    // fp32 outputs are stored non-temporally
 };
 
 

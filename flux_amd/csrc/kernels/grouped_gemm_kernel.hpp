@@ -139,6 +139,7 @@ __device__ __forceinline__ void store_tile(uint8_t *windows, const TileCtx &c, i
   const int64_t rowgroup_bytes = static_cast<int64_t>(8) * n * ELT_OUT;
   const int32_t *scatter = FULL ? nullptr : p->scatter_d;
   const int max_rows = p->max_rows;
+  const bool nt_stores = p->nt_stores != 0;  // wave-uniform
   int block = 0;
 #pragma unroll
   for (int j = 0; j < NB; ++j) {
@@ -190,7 +191,13 @@ __device__ __forceinline__ void store_tile(uint8_t *windows, const TileCtx &c, i
         float4 o = v[it];
         if constexpr (SCALED) o = make_float4(o.x * cs.x, o.y * cs.y, o.z * cs.z, o.w * cs.w);
         if constexpr (OUT_F32) {
-          *reinterpret_cast<float4 *>(dst) = o;
+          if (nt_stores) {
+            typedef float f32x4_t __attribute__((ext_vector_type(4)));
+            const f32x4_t ov = {o.x, o.y, o.z, o.w};
+            __builtin_nontemporal_store(ov, reinterpret_cast<f32x4_t *>(dst));
+          } else {
+            *reinterpret_cast<float4 *>(dst) = o;
+          }
         } else {
           u32x2 b;
           b[0] = pack_bf16x2(o.x, o.y);
