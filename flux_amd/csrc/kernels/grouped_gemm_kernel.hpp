@@ -9,6 +9,7 @@ namespace {
 #define FLUXMI_WAITCNT(vm, lgkm) \
   __builtin_amdgcn_s_waitcnt(((vm)&15) | (((vm) >> 4) << 14) | (7 << 4) | ((lgkm) << 8))
 
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) void *lds_ptr_t;
 typedef const __attribute__((address_space(1))) void *gbl_ptr_t;
 
@@ -140,6 +141,57 @@ __device__ __forceinline__ void store_tile(uint8_t *windows, const TileCtx &c, i
   const int32_t *scatter = FULL ? nullptr : p->scatter_d;
   const int max_rows = p->max_rows;
   const bool nt_stores = p->nt_stores != 0;  // wave-uniform
+  if constexpr (ELT == 2 && !OUT_F32 && FULL && NB % 2 == 0) {
+    // bf16 rows of whole tiles leave as whole 128-byte lines: two 32-column blocks per pass, packed to bf16
+    // before the pass, so that the window (64 rows x 128 bytes) comes back as eight lanes x 16 bytes per row.
+    // In 64-byte pieces a line is written in two halves at different times and part of the lines reach HBM
+    // twice.  Needs 16-byte aligned rows; other outputs take the 64-byte path below.
+    if ((n & 7) == 0 && (reinterpret_cast<uintptr_t>(d) & 15u) == 0) {
+      uint8_t *const wlane = d + (static_cast<int64_t>(row_base + wrow0 + rr0) * n + wcol0 + cc * 8) * 2;
+#pragma unroll
+      for (int j2 = 0; j2 < NB / 2; ++j2) {
+#pragma unroll
+        for (int ip = 0; ip < MB / 2; ++ip) {
+          uint8_t *window = windows;
+#pragma unroll
+          for (int jq = 0; jq < 4; ++jq) {
+            const int jb = j2 * 4 + jq;
+            float4 cs = make_float4(1.f, 1.f, 1.f, 1.f);
+            if constexpr (SCALED) {
+              if (col_scale)
+                cs = *reinterpret_cast<const float4 *>(col_scale + static_cast<int64_t>(e) * n + wcol0 + jb * 16 + 4 * (lane >> 4));
+            }
+#pragma unroll
+            for (int ii = 0; ii < 4; ++ii) {
+              const int i = ip * 4 + ii;
+              const int r = ii * 16 + (lane & 15);
+              float4 v = make_float4(acc_read(acc[i][jb][0]), acc_read(acc[i][jb][1]), acc_read(acc[i][jb][2]),
+                                     acc_read(acc[i][jb][3]));
+              if constexpr (SCALED) {
+                v = make_float4(v.x * rs[i], v.y * rs[i], v.z * rs[i], v.w * rs[i]);
+                v = make_float4(v.x * cs.x, v.y * cs.y, v.z * cs.z, v.w * cs.w);
+              }
+              u32x2 b;
+              b[0] = pack_bf16x2(v.x, v.y);
+              b[1] = pack_bf16x2(v.z, v.w);
+              const int chunk = jq * 2 + (lane >> 5);  // 16-byte chunk of the 128-byte row; (lane >> 4) & 1: its half
+              *reinterpret_cast<u32x2 *>(window + r * 128 + ((chunk ^ ((r >> 1) & 7)) << 4) + ((lane >> 4) & 1) * 8) = b;
+            }
+          }
+          u32x4 v[8];
+#pragma unroll
+          for (int it = 0; it < 8; ++it) {
+            const int rr = it * 8 + rr0;
+            v[it] = *reinterpret_cast<const u32x4 *>(window + rr * 128 + ((cc ^ ((rr >> 1) & 7)) << 4));
+          }
+          uint8_t *dp = wlane + (static_cast<int64_t>(ip) * 8) * rowgroup_bytes + j2 * 128;
+#pragma unroll
+          for (int it = 0; it < 8; ++it, dp += rowgroup_bytes) *reinterpret_cast<u32x4 *>(dp) = v[it];
+        }
+      }
+      return;
+    }
+  }
   int block = 0;
 #pragma unroll
   for (int j = 0; j < NB; ++j) {
