@@ -3,8 +3,9 @@
   libfluxmi_kernels.so   HIP kernels + C-ABI (include/fluxmi.h)       <- flux_amd/csrc/kernels/*.hip
   flux_ths_pybind*.so    C++ torch extension with Flux's op surface    <- flux_amd/csrc/ths_op/*.cc
 
-Usage: python -m flux_amd.build [--kernels-only] [--force]
-Outputs land in flux_amd/lib/ and travel with the source tree; nothing is installed.
+Usage: python -m flux_amd.build [--kernels-only] [--no-force]
+Everything is rebuilt unless --no-force is given; with it, only translation units older than a file they
+include are compiled again.  Outputs land in flux_amd/lib/ and travel with the source tree; nothing is installed.
 """
 import argparse
 import concurrent.futures
@@ -48,21 +49,43 @@ def _newer(target, sources):
     return all(os.path.getmtime(s) <= t for s in sources)
 
 
+def _deps_of(depfile):
+    """Prerequisites listed in a make-style dependency file written by the compiler (-MD -MF)."""
+    try:
+        text = open(depfile).read()
+    except OSError:
+        return None
+    text = text.replace("\\\n", " ")
+    _, _, rhs = text.partition(":")
+    return [t for t in rhs.split() if t]
+
+
+def _object_current(obj, depfile):
+    deps = _deps_of(depfile)
+    if deps is None or not os.path.exists(obj):
+        return False
+    t = os.path.getmtime(obj)
+    return all(os.path.exists(d) and os.path.getmtime(d) <= t for d in deps)
+
+
 def build_kernels(force=True):
     os.makedirs(OBJ_DIR, exist_ok=True)
     srcs = sorted(f for f in os.listdir(KERNEL_DIR) if f.endswith(".hip"))
-    deps = [os.path.join(KERNEL_DIR, f) for f in os.listdir(KERNEL_DIR)] + [os.path.join(INCLUDE, "fluxmi.h")]
-    if not force and _newer(KERNEL_LIB, deps):
-        return KERNEL_LIB
+    rebuilt = []
 
     def compile_one(name):
         obj = os.path.join(OBJ_DIR, name[:-4] + ".o")
-        _run([HIPCC, *HIP_FLAGS, "-c", os.path.join(KERNEL_DIR, name), "-o", obj])
+        dep = obj[:-2] + ".d"
+        if not force and _object_current(obj, dep):
+            return obj
+        _run([HIPCC, *HIP_FLAGS, "-MD", "-MF", dep, "-c", os.path.join(KERNEL_DIR, name), "-o", obj])
+        rebuilt.append(name)
         return obj
 
     with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(srcs))) as pool:
         objs = list(pool.map(compile_one, srcs))
-    _run([HIPCC, f"--offload-arch={ARCH}", "-shared", "-fPIC", *objs, "-o", KERNEL_LIB])
+    if rebuilt or not os.path.exists(KERNEL_LIB):
+        _run([HIPCC, f"--offload-arch={ARCH}", "-shared", "-fPIC", *objs, "-o", KERNEL_LIB])
     return KERNEL_LIB
 
 

@@ -18,7 +18,8 @@ FP8_E4M3 = 1
 EXPORTS = (
     "fluxmi_version", "fluxmi_last_error", "fluxmi_device_cu_count",
     "fluxmi_moe_route_sort_workspace_bytes", "fluxmi_moe_route_sort", "fluxmi_moe_gather_index",
-    "fluxmi_grouped_gemm_workspace_bytes", "fluxmi_grouped_gemm", "fluxmi_grouped_gemm_multi",
+    "fluxmi_grouped_gemm_workspace_bytes", "fluxmi_grouped_gemm", "fluxmi_grouped_gemm_kernel_kind",
+    "fluxmi_grouped_gemm_multi",
     "fluxmi_topk_gather_reduce", "fluxmi_quant_e4m3_rowwise", "fluxmi_quant_e4m3_square",
     "fluxmi_quant_e4m3_block128",
 )
@@ -62,6 +63,7 @@ def load():
     lib.fluxmi_grouped_gemm_workspace_bytes.restype = sz
     lib.fluxmi_grouped_gemm_workspace_bytes.argtypes = [ctypes.POINTER(GroupedGemmArgs)]
     lib.fluxmi_grouped_gemm.argtypes = [ctypes.POINTER(GroupedGemmArgs), vp, sz, vp]
+    lib.fluxmi_grouped_gemm_kernel_kind.argtypes = [ctypes.POINTER(GroupedGemmArgs)]
     lib.fluxmi_grouped_gemm_multi.argtypes = [ctypes.POINTER(GroupedGemmArgs), i32, vp, vp, vp, vp, sz, vp]
     lib.fluxmi_topk_gather_reduce.argtypes = [ctypes.POINTER(vp), i32, i32, vp, vp, f32, i32, i32, i32, vp, vp]
     lib.fluxmi_quant_e4m3_rowwise.argtypes = [vp, i64, i64, i32, f32, vp, vp, i32, vp]
@@ -128,8 +130,9 @@ SCHED_NO_HALF_TILES = 2
 
 def grouped_gemm(a, b, splits, out=None, gather_a=None, scatter_d=None, alpha=None, row_scale=None,
                  col_scale=None, scalar_scale=1.0, scalar_scale_dev=None, max_rows=None, out_dtype=None,
-                 cu_margin=0, raster_rows=0, sched_flags=0):
-    """D = grouped GEMM of A [rows_a, K] with B [E, N, K]; see fluxmi_grouped_gemm in include/fluxmi.h."""
+                 cu_margin=0, raster_rows=0, sched_flags=0, want_kind=False):
+    """D = grouped GEMM of A [rows_a, K] with B [E, N, K]; see fluxmi_grouped_gemm in include/fluxmi.h.
+    With `want_kind` the result is (D, kind): kind 1 = the MFMA kernel ran, 0 = the generic kernel."""
     lib = load()
     if a.dtype == torch.bfloat16:
         dtype = BF16
@@ -169,6 +172,8 @@ def grouped_gemm(a, b, splits, out=None, gather_a=None, scatter_d=None, alpha=No
         scalar_scale_dev=None if scalar_scale_dev is None else scalar_scale_dev.data_ptr(),
         cu_margin=cu_margin, raster_rows=raster_rows, sched_flags=sched_flags)
     _check(lib.fluxmi_grouped_gemm(ctypes.byref(args), None, 0, _stream()), "fluxmi_grouped_gemm")
+    if want_kind:
+        return out, lib.fluxmi_grouped_gemm_kernel_kind(ctypes.byref(args))
     return out
 
 

@@ -71,6 +71,12 @@ __device__ __forceinline__ void accumulate8(float (&acc)[8], const Vec8<false> &
   }
 }
 
+// A routing entry names a source row only inside [0, nrows): negative entries mark dropped pairs, and an
+// entry at or past the end of the input must never be dereferenced.
+__device__ __forceinline__ bool row_in_range(int32_t r, int32_t nrows) {
+  return static_cast<uint32_t>(r) < static_cast<uint32_t>(nrows);
+}
+
 __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
   return static_cast<uint32_t>(float_to_bf16_bits(lo)) | (static_cast<uint32_t>(float_to_bf16_bits(hi)) << 16);
 }
@@ -81,7 +87,7 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
 template <int TOPK, int NGROUPS, bool WEIGHTED, bool IN_F32, bool NT>
 __device__ __forceinline__ void topk_gather_reduce_body(
     const GroupPtrs &in, const int32_t *__restrict__ routing_idx, const float *__restrict__ row_weight,
-    float scale, int32_t topk_rt, int32_t nvec, uint16_t *__restrict__ out) {
+    float scale, int32_t topk_rt, int32_t nvec, int32_t nrows, uint16_t *__restrict__ out) {
   const int t = blockIdx.x;
   const int topk = TOPK > 0 ? TOPK : topk_rt;
   const size_t row_vecs = static_cast<size_t>(nvec);
@@ -98,15 +104,16 @@ __device__ __forceinline__ void topk_gather_reduce_body(
 #pragma unroll
       for (int j = 0; j < TOPK; ++j) {
         const int32_t r = routing_idx[static_cast<size_t>(t) * TOPK + j];
+        const bool live = row_in_range(r, nrows);
         w[j] = 0.f;
-        if (r >= 0) w[j] = WEIGHTED ? row_weight[r] : 1.f;
+        if (live) w[j] = WEIGHTED ? row_weight[r] : 1.f;
 #pragma unroll
         for (int g = 0; g < NGROUPS; ++g) {
           va[g][j] = u32x4{0u, 0u, 0u, 0u};
           vb[g][j] = u32x4{0u, 0u, 0u, 0u};
-          const u32x4 *src = reinterpret_cast<const u32x4 *>(in.p[g]) + static_cast<size_t>(r < 0 ? 0 : r) * nq;
-          if (r >= 0 && oka) va[g][j] = load16<NT>(src + qa);
-          if (r >= 0 && okb) vb[g][j] = load16<NT>(src + qb);
+          const u32x4 *src = reinterpret_cast<const u32x4 *>(in.p[g]) + static_cast<size_t>(live ? r : 0) * nq;
+          if (live && oka) va[g][j] = load16<NT>(src + qa);
+          if (live && okb) vb[g][j] = load16<NT>(src + qb);
         }
       }
       float a[4] = {0.f, 0.f, 0.f, 0.f}, b[4] = {0.f, 0.f, 0.f, 0.f};
@@ -146,13 +153,14 @@ __device__ __forceinline__ void topk_gather_reduce_body(
 #pragma unroll
       for (int j = 0; j < TOPK; ++j) {
         const int32_t r = routing_idx[static_cast<size_t>(t) * TOPK + j];
+        const bool live = row_in_range(r, nrows);
         w[j] = 0.f;
-        if (r >= 0) w[j] = WEIGHTED ? row_weight[r] : 1.f;
+        if (live) w[j] = WEIGHTED ? row_weight[r] : 1.f;
 #pragma unroll
         for (int g = 0; g < NGROUPS; ++g) {
           vals[g][j] = zero8<IN_F32>();
-          // r is wave-uniform: a skipped (dropped) row costs no traffic
-          if (r >= 0) vals[g][j] = load8<IN_F32, NT>(in.p[g], static_cast<size_t>(r), row_vecs, v);
+          // r is wave-uniform: a skipped (dropped or out-of-range) row costs no traffic
+          if (live) vals[g][j] = load8<IN_F32, NT>(in.p[g], static_cast<size_t>(r), row_vecs, v);
         }
       }
 #pragma unroll
@@ -164,7 +172,7 @@ __device__ __forceinline__ void topk_gather_reduce_body(
       for (int g = 0; g < NGROUPS; ++g) {
         for (int j = 0; j < topk; ++j) {
           const int32_t r = routing_idx[static_cast<size_t>(t) * topk + j];
-          if (r < 0) continue;
+          if (!row_in_range(r, nrows)) continue;
           const float w = WEIGHTED ? row_weight[r] : 1.f;
           accumulate8(acc, load8<IN_F32, NT>(in.p[g], static_cast<size_t>(r), row_vecs, v), w);
         }
@@ -185,22 +193,22 @@ __device__ __forceinline__ void topk_gather_reduce_body(
 template <int TOPK, int NGROUPS, bool WEIGHTED, bool IN_F32>
 __global__ __launch_bounds__(kMaxThreads) void topk_gather_reduce_kernel(
     GroupPtrs in, const int32_t *__restrict__ routing_idx, const float *__restrict__ row_weight,
-    float scale, int32_t topk_rt, int32_t nvec /* n / 8 */, int32_t nt_loads,
+    float scale, int32_t topk_rt, int32_t nvec /* n / 8 */, int32_t nrows, int32_t nt_loads,
     uint16_t *__restrict__ out) {
   if (nt_loads)
     topk_gather_reduce_body<TOPK, NGROUPS, WEIGHTED, IN_F32, true>(in, routing_idx, row_weight, scale, topk_rt,
-                                                                   nvec, out);
+                                                                   nvec, nrows, out);
   else
     topk_gather_reduce_body<TOPK, NGROUPS, WEIGHTED, IN_F32, false>(in, routing_idx, row_weight, scale, topk_rt,
-                                                                    nvec, out);
+                                                                    nvec, nrows, out);
 }
 
 template <int TOPK, int NGROUPS>
 void launch(bool weighted, bool in_f32, dim3 grid, int threads, int nt, hipStream_t s, const GroupPtrs &in,
-            const int32_t *idx, const float *w, float scale, int32_t topk, int32_t nvec, uint16_t *out) {
+            const int32_t *idx, const float *w, float scale, int32_t topk, int32_t nvec, int32_t nrows, uint16_t *out) {
 #define FLUXMI_GR_LAUNCH(W, F)                                                                       \
   hipLaunchKernelGGL((topk_gather_reduce_kernel<TOPK, NGROUPS, W, F>), grid, dim3(threads), 0, s, in, \
-                     idx, w, scale, topk, nvec, nt, out)
+                     idx, w, scale, topk, nvec, nrows, nt, out)
   if (weighted) {
     if (in_f32) FLUXMI_GR_LAUNCH(true, true);
     else FLUXMI_GR_LAUNCH(true, false);
@@ -213,14 +221,14 @@ void launch(bool weighted, bool in_f32, dim3 grid, int threads, int nt, hipStrea
 
 template <int NGROUPS>
 void dispatch_topk(bool weighted, bool in_f32, dim3 grid, int threads, int nt, hipStream_t s, const GroupPtrs &in, const int32_t *idx,
-                   const float *w, float scale, int32_t topk, int32_t nvec, uint16_t *out) {
+                   const float *w, float scale, int32_t topk, int32_t nvec, int32_t nrows, uint16_t *out) {
   switch (topk) {
-    case 1: launch<1, NGROUPS>(weighted, in_f32, grid, threads, nt, s, in, idx, w, scale, topk, nvec, out); break;
-    case 2: launch<2, NGROUPS>(weighted, in_f32, grid, threads, nt, s, in, idx, w, scale, topk, nvec, out); break;
-    case 4: launch<4, NGROUPS>(weighted, in_f32, grid, threads, nt, s, in, idx, w, scale, topk, nvec, out); break;
-    case 6: launch<6, NGROUPS>(weighted, in_f32, grid, threads, nt, s, in, idx, w, scale, topk, nvec, out); break;
-    case 8: launch<8, NGROUPS>(weighted, in_f32, grid, threads, nt, s, in, idx, w, scale, topk, nvec, out); break;
-    default: launch<0, NGROUPS>(weighted, in_f32, grid, threads, nt, s, in, idx, w, scale, topk, nvec, out); break;
+    case 1: launch<1, NGROUPS>(weighted, in_f32, grid, threads, nt, s, in, idx, w, scale, topk, nvec, nrows, out); break;
+    case 2: launch<2, NGROUPS>(weighted, in_f32, grid, threads, nt, s, in, idx, w, scale, topk, nvec, nrows, out); break;
+    case 4: launch<4, NGROUPS>(weighted, in_f32, grid, threads, nt, s, in, idx, w, scale, topk, nvec, nrows, out); break;
+    case 6: launch<6, NGROUPS>(weighted, in_f32, grid, threads, nt, s, in, idx, w, scale, topk, nvec, nrows, out); break;
+    case 8: launch<8, NGROUPS>(weighted, in_f32, grid, threads, nt, s, in, idx, w, scale, topk, nvec, nrows, out); break;
+    default: launch<0, NGROUPS>(weighted, in_f32, grid, threads, nt, s, in, idx, w, scale, topk, nvec, nrows, out); break;
   }
 }
 
@@ -253,6 +261,9 @@ extern "C" int fluxmi_topk_gather_reduce(const void *const *in, int32_t ngroups,
   if (ntokens == 0 || n == 0) return FLUXMI_OK;
 
   const int32_t nvec = n / 8;
+  FLUXMI_REQUIRE(static_cast<int64_t>(ntokens) * topk <= INT32_MAX, FLUXMI_ERR_UNSUPPORTED,
+                 "topk_gather_reduce: ntokens*topk exceeds 2^31-1");
+  const int32_t nrows = ntokens * topk;  // rows of every input matrix
   // One workgroup per token row; rows wider than 2 vectors per lane are split over blockIdx.y so
   // that small token counts still fill the chip.
   const int threads = nvec >= 512 ? 512 : 256;
@@ -268,10 +279,10 @@ extern "C" int fluxmi_topk_gather_reduce(const void *const *in, int32_t ngroups,
   const bool weighted = row_weight != nullptr;
   uint16_t *o = static_cast<uint16_t *>(out);
   switch (ngroups) {
-    case 1: dispatch_topk<1>(weighted, in_fp32 != 0, grid, threads, nt, s, gp, routing_idx, row_weight, scale, topk, nvec, o); break;
-    case 2: dispatch_topk<2>(weighted, in_fp32 != 0, grid, threads, nt, s, gp, routing_idx, row_weight, scale, topk, nvec, o); break;
-    case 3: dispatch_topk<3>(weighted, in_fp32 != 0, grid, threads, nt, s, gp, routing_idx, row_weight, scale, topk, nvec, o); break;
-    default: dispatch_topk<4>(weighted, in_fp32 != 0, grid, threads, nt, s, gp, routing_idx, row_weight, scale, topk, nvec, o); break;
+    case 1: dispatch_topk<1>(weighted, in_fp32 != 0, grid, threads, nt, s, gp, routing_idx, row_weight, scale, topk, nvec, nrows, o); break;
+    case 2: dispatch_topk<2>(weighted, in_fp32 != 0, grid, threads, nt, s, gp, routing_idx, row_weight, scale, topk, nvec, nrows, o); break;
+    case 3: dispatch_topk<3>(weighted, in_fp32 != 0, grid, threads, nt, s, gp, routing_idx, row_weight, scale, topk, nvec, nrows, o); break;
+    default: dispatch_topk<4>(weighted, in_fp32 != 0, grid, threads, nt, s, gp, routing_idx, row_weight, scale, topk, nvec, nrows, o); break;
   }
   FLUXMI_HIP_CHECK(hipGetLastError());
   return FLUXMI_OK;

@@ -71,15 +71,16 @@ __global__ __launch_bounds__(256) void grouped_gemm_generic_kernel(const GemmPar
   }
 }
 
-// Shapes the MFMA kernel takes: K a multiple of 64 bytes, N a multiple of 4, aligned pointers, and
-// operands its 32-bit buffer offsets can span (a gathered A as a whole, 256 rows of an ungathered A, one
-// expert's weights).  Everything else runs the generic kernel.
+// Shapes the MFMA kernel takes: rows of K a multiple of 16 bytes (K % 8 == 0 for bf16, K % 16 == 0 for fp8),
+// N a multiple of 4, aligned pointers, and operands its 32-bit buffer offsets can span (a gathered A as a
+// whole, which needs its extent a_rows; 256 rows of an ungathered A; one expert's weights).  Everything else
+// runs the generic kernel.
 bool mfma_path_ok(const fluxmi_grouped_gemm_args *a, const void *b, const void *d) {
   const int elt = a->dtype == FLUXMI_BF16 ? 2 : 1;
   const int64_t kbytes = static_cast<int64_t>(a->k) * elt;
   const int64_t span = 0xffffffffll;
   const bool a_fits = a->gather_a ? (a->a_rows > 0 && a->a_rows * kbytes <= span) : BM * kbytes <= span;
-  return kbytes % KBYTES == 0 && kbytes >= KBYTES && a->n % 4 == 0 && aligned16(a->a) &&
+  return kbytes % 16 == 0 && kbytes >= 16 && a->n % 4 == 0 && aligned16(a->a) &&
          aligned16(b) && (reinterpret_cast<uintptr_t>(d) & (a->d_fp32 ? 15u : 7u)) == 0 &&
          (a->col_scale == nullptr || aligned16(a->col_scale)) && a_fits && a->n * kbytes <= span;
 }
@@ -92,14 +93,17 @@ extern "C" size_t fluxmi_grouped_gemm_workspace_bytes(const fluxmi_grouped_gemm_
 namespace fluxmi {
 namespace {
 
+// dry_run: check the arguments and report which kernel would run (1 MFMA, 0 generic) without launching.
 int run_grouped_gemm(const fluxmi_grouped_gemm_args *args, int ngroups, const void *const *b, void *const *d,
-                     const float *const *alpha, void *stream) {
+                     const float *const *alpha, void *stream, bool dry_run = false) {
   FLUXMI_REQUIRE(args != nullptr, FLUXMI_ERR_INVALID_ARG, "grouped_gemm: null args");
   FLUXMI_REQUIRE(args->dtype == FLUXMI_BF16 || args->dtype == FLUXMI_FP8_E4M3, FLUXMI_ERR_INVALID_ARG,
                  "grouped_gemm: unknown dtype %d", args->dtype);
   FLUXMI_REQUIRE(args->d_fp32 == 0 || args->d_fp32 == 1, FLUXMI_ERR_INVALID_ARG,
                  "grouped_gemm: d_fp32 must be 0 or 1");
   FLUXMI_REQUIRE(args->a_rows >= 0, FLUXMI_ERR_INVALID_ARG, "grouped_gemm: negative a_rows");
+  FLUXMI_REQUIRE(args->reserved == 0, FLUXMI_ERR_INVALID_ARG, "grouped_gemm: reserved must be 0, got %d",
+                 args->reserved);
   FLUXMI_REQUIRE(args->nexperts >= 1 && args->nexperts <= kMaxExperts, FLUXMI_ERR_UNSUPPORTED,
                  "grouped_gemm: nexperts=%d outside [1,%d]", args->nexperts, kMaxExperts);
   FLUXMI_REQUIRE(args->max_rows >= 0 && args->n >= 0 && args->k >= 0, FLUXMI_ERR_INVALID_ARG,
@@ -107,7 +111,7 @@ int run_grouped_gemm(const fluxmi_grouped_gemm_args *args, int ngroups, const vo
                  args->k);
   FLUXMI_REQUIRE(ngroups >= 1 && ngroups <= kMaxWeightGroups, FLUXMI_ERR_UNSUPPORTED,
                  "grouped_gemm: ngroups=%d outside [1,%d]", ngroups, kMaxWeightGroups);
-  if (args->max_rows == 0 || args->n == 0) return FLUXMI_OK;
+  if (args->max_rows == 0 || args->n == 0) return dry_run ? 1 : FLUXMI_OK;
   FLUXMI_REQUIRE(args->k >= 1, FLUXMI_ERR_UNSUPPORTED, "grouped_gemm: k must be positive");
   FLUXMI_REQUIRE(args->a && args->splits && b && d, FLUXMI_ERR_INVALID_ARG, "grouped_gemm: null a / b / d / splits");
 
@@ -149,6 +153,7 @@ int run_grouped_gemm(const fluxmi_grouped_gemm_args *args, int ngroups, const vo
   p.raster_rows = args->raster_rows > 0 ? args->raster_rows : 8;
   p.sched_flags = args->sched_flags;
 
+  if (dry_run) return mfma ? 1 : 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   int cus = fluxmi_device_cu_count();
   FLUXMI_REQUIRE(cus > 0, FLUXMI_ERR_HIP, "grouped_gemm: cannot query the device");
@@ -184,6 +189,14 @@ extern "C" int fluxmi_grouped_gemm(const fluxmi_grouped_gemm_args *args, void *,
   void *d = args->d;
   const float *alpha = args->alpha;
   return fluxmi::run_grouped_gemm(args, 1, &b, &d, &alpha, stream);
+}
+
+extern "C" int fluxmi_grouped_gemm_kernel_kind(const fluxmi_grouped_gemm_args *args) {
+  FLUXMI_REQUIRE(args != nullptr, FLUXMI_ERR_INVALID_ARG, "grouped_gemm: null args");
+  const void *b = args->b;
+  void *d = args->d;
+  const float *alpha = args->alpha;
+  return fluxmi::run_grouped_gemm(args, 1, &b, &d, &alpha, nullptr, /*dry_run=*/true);
 }
 
 extern "C" int fluxmi_grouped_gemm_multi(const fluxmi_grouped_gemm_args *args, int32_t ngroups, const void *const *b,

@@ -81,7 +81,9 @@ struct TileCtx {
   int wave, lane, wn, wm;
   int fill_row, fill_chunk;
   int frag_off[2];
-  int nk;
+  int nk;           // k-steps of 64 bytes per row, a partial last one included
+  int nkf;          // whole k-steps
+  int tail_chunks;  // 16-byte chunks of the partial last k-step (0: K is a whole number of k-steps)
   int64_t kbytes;
   float scalar;
 };
@@ -357,6 +359,20 @@ __device__ __forceinline__ void setup_operands(const GemmParams &p, const TileCt
   }
 }
 
+// The partial last k-step of a K that is not a whole number of k-steps: lanes whose 16-byte chunk lies inside
+// the row fetch it, the others write zeros to their LDS slot themselves (an out-of-range direct-to-LDS load
+// writes nothing).  Still one vector-memory instruction per wave, so the fill counts of the waits hold; the
+// LDS write is waited for on the spot (a rare path: once per operand row group and tile).
+__device__ __forceinline__ void fill_partial(__amdgpu_buffer_rsrc_t rsrc, uint32_t off, int kbyte, uint8_t *dst,
+                                             const TileCtx &c) {
+  if (c.fill_chunk < c.tail_chunks) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)dst, 16, static_cast<int>(off), kbyte, 0, 0);
+  } else {
+    *reinterpret_cast<u32x4 *>(dst + c.lane * 16) = u32x4{0u, 0u, 0u, 0u};
+  }
+  FLUXMI_WAITCNT(63, 0);
+}
+
 // Fill instruction q (X rows first, then W rows) of k-step `kstep` of a tile into ring slot `slot`.  A
 // k-step past the end of K (the phantom second half of the last pair of an odd K) is filled from the
 // zero page.  The k offset travels as the scalar offset: an instruction immediate would also be added
@@ -364,16 +380,22 @@ __device__ __forceinline__ void setup_operands(const GemmParams &p, const TileCt
 template <int XL, int WL>
 __device__ __forceinline__ void fill_any(const TileOperands<XL, WL> &op, uint8_t *smem, const TileCtx &c, int q, int slot,
                                          int kstep) {
-  const bool in = kstep < c.nk;
+  const bool in = kstep < c.nkf;
   const int kbyte = in ? kstep * KBYTES : 0;
   const __amdgpu_buffer_rsrc_t zrsrc = make_rsrc(g_zero_page, 1024);
   const uint32_t zoff = c.lane * 16;
+  uint8_t *const dst = q < XL ? smem + slot * Ring<XL, WL>::SB + (XL * c.wave + q) * 1024
+                              : smem + slot * Ring<XL, WL>::SB + Ring<XL, WL>::XB + (WL * c.wave + (q - XL)) * 1024;
+  if (kstep == c.nkf && c.tail_chunks != 0) {  // wave-uniform
+    if (q < XL) fill_partial(op.xrsrc, op.xoff[q < XL ? q : 0], kstep * KBYTES, dst, c);
+    else fill_partial(op.wrsrc, op.woff[q >= XL ? q - XL : 0], kstep * KBYTES, dst, c);
+    return;
+  }
   if (q < XL)
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(in ? op.xrsrc : zrsrc, (lds_ptr_t)(smem + slot * Ring<XL, WL>::SB + (XL * c.wave + q) * 1024), 16,
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(in ? op.xrsrc : zrsrc, (lds_ptr_t)dst, 16,
                                              static_cast<int>(in ? op.xoff[q < XL ? q : 0] : zoff), kbyte, 0, 0);
   else
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(in ? op.wrsrc : zrsrc,
-                                             (lds_ptr_t)(smem + slot * Ring<XL, WL>::SB + Ring<XL, WL>::XB + (WL * c.wave + (q - XL)) * 1024), 16,
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(in ? op.wrsrc : zrsrc, (lds_ptr_t)dst, 16,
                                              static_cast<int>(in ? op.woff[q >= XL ? q - XL : 0] : zoff), kbyte, 0, 0);
 }
 
@@ -452,7 +474,9 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
   auto fill_m0 = [&](auto SLOT, auto Q) {
     constexpr int slot = decltype(SLOT)::value, q = decltype(Q)::value;
     const uint32_t dst = q < XLOADS ? xdst32 + slot * SB + q * 1024 : wdst32 + slot * SB + (q - XLOADS) * 1024;
-    asm volatile("s_mov_b32 m0, %0" : : "s"(dst) : "memory");
+    // M0 is declared clobbered so that the compiler never assumes a value it wrote to M0 earlier (for a fill it
+    // emitted itself) is still there after this statement.
+    asm volatile("s_mov_b32 m0, %0" : : "s"(dst) : "memory", "m0");
   };
   auto fill_go = [&](auto Q, int kbyte) {
     constexpr int q = decltype(Q)::value;
@@ -468,10 +492,16 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
   };
   // Same with a run-time slot, for the last steps of a tile; a k-step past the end of K (the phantom
   // second half of the last pair of an odd K) is filled from the zero page.
+  const int nkf = c.nkf;
   auto fill_dyn = [&](int slot, auto Q, int kstep) {
     constexpr int q = decltype(Q)::value;
-    const bool in = kstep < nk;
+    const bool in = kstep < nkf;
     const int kbyte = in ? kstep * KBYTES : 0;
+    if (kstep == nkf && c.tail_chunks != 0) {  // the partial last k-step (wave-uniform branch)
+      if constexpr (q < XLOADS) fill_partial(xrsrc, xoff[q], kstep * KBYTES, xdst + slot * SB + q * 1024, c);
+      else fill_partial(wrsrc, woff[q - XLOADS], kstep * KBYTES, wdst + slot * SB + (q - XLOADS) * 1024, c);
+      return;
+    }
     if constexpr (q < XLOADS)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(in ? xrsrc : zrsrc, (lds_ptr_t)(xdst + slot * SB + q * 1024), 16,
                                                static_cast<int>(in ? xoff[q] : zoff), kbyte, 0, 0);
@@ -608,10 +638,10 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
   FLUXMI_WAITCNT(63, 0);  // in registers before the first step's barrier lets anyone refill that slot
 
   // ---- main loop ----------------------------------------------------------------------------------
-  // Whole trips of ten k-steps while every k-step a trip requests (up to 9 + LA past its first one) exists,
-  // then the remaining steps pair by pair with run-time ring slots.  An odd number of k-steps
+  // Whole trips of ten k-steps while every k-step a trip requests (up to 9 + LA past its first one) is a whole
+  // one, then the remaining steps pair by pair with run-time ring slots.  An odd number of k-steps
   // ends with a phantom step on zero fragments.
-  const int nfast = nk >= 10 + LA ? (nk - (10 + LA)) / 10 + 1 : 0;  // trips with 10 * trip + 9 + LA < nk
+  const int nfast = nkf >= 10 + LA ? (nkf - (10 + LA)) / 10 + 1 : 0;  // trips with 10 * trip + 9 + LA < nkf
   int kbase = 0;  // byte offset along K of step 0 of the current trip
   for (int trip = 0; trip < nfast; ++trip) {
     step(std::integral_constant<int, 0>{}, kbase, xa, wa, xb, wb);
@@ -680,7 +710,9 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
   const int tiles_n1 = (p.n + BN - 1) / BN;  // column tiles of one weight group
   const int tiles_n = tiles_n1 * p.ngroups;  // ... of the launch
   c.kbytes = static_cast<int64_t>(p.k) * ELT;
-  c.nk = static_cast<int>(c.kbytes / KBYTES);
+  c.nkf = static_cast<int>(c.kbytes / KBYTES);
+  c.tail_chunks = static_cast<int>(c.kbytes % KBYTES) / 16;
+  c.nk = c.nkf + (c.tail_chunks != 0 ? 1 : 0);
 
   // LDS tile layout: rows of 64 bytes = four 16-byte chunks; a direct-to-LDS fill instruction covers 16
   // rows = 1 KiB, lane l landing at byte 16 * l of it, so which (row, chunk) a slot holds is decided by the

@@ -23,41 +23,17 @@ __device__ __forceinline__ float compute_scale(float amax, float eps) {
   return s;  // includes s == 0 when amax is +inf
 }
 
-#ifdef FLUXMI_SOFT_FP8
-// Bit-level fp32 -> e4m3 (OCP "fn"): round to nearest even, saturate to +-448, NaN -> 0x7f.
-__device__ __forceinline__ uint32_t f32_to_e4m3(float f) {
-  const uint32_t u = __float_as_uint(f);
-  const uint32_t sign = (u >> 24) & 0x80u;
-  uint32_t a = u & 0x7fffffffu;
-  if (a > 0x7f800000u) return sign | 0x7fu;
-  if (a >= 0x43e00000u) return sign | 0x7eu;  // |f| >= 448
-  if (a < 0x3c800000u) {                      // |f| < 2^-6: subnormal grid of 2^-9
-    const float q = __builtin_rintf(__uint_as_float(a) * 512.f);
-    return sign | static_cast<uint32_t>(q);
-  }
-  a += 0x7ffffu + ((a >> 20) & 1u);
-  return sign | ((a >> 20) - (120u << 3));
-}
-__device__ __forceinline__ uint32_t pack2_e4m3(float lo, float hi) {
-  return f32_to_e4m3(lo) | (f32_to_e4m3(hi) << 8);
-}
-#else
 // Hardware conversion (v_cvt_pk_fp8_f32, OCP e4m3 on gfx950, round to nearest even).  The operands are
 // clamped first so that the result saturates whatever the conversion's own overflow rule is; NaN
 // passes through the clamp untouched.
 __device__ __forceinline__ float clamp448(float f) {
-#ifdef FLUXMI_NO_CLAMP
-  return f;
-#else
   const float c = fminf(fmaxf(f, -kE4M3Max), kE4M3Max);
   return f != f ? f : c;
-#endif
 }
 __device__ __forceinline__ uint32_t pack2_e4m3(float lo, float hi) {
   return static_cast<uint32_t>(__builtin_amdgcn_cvt_pk_fp8_f32(clamp448(lo), clamp448(hi), 0, false)) &
          0xffffu;
 }
-#endif
 
 // Largest |x| of 8 bf16 values as fp32 bits.  Done on the integer patterns (for non-negative floats the
 // unsigned order is the numeric order) so that every NaN, signalling ones included, is skipped exactly

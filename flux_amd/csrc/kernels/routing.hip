@@ -2,14 +2,16 @@
 // gather_index, topk_index.
 //
 // The flat pair array is cut into chunks of kChunk = 512 pairs, one wave per chunk (8 wave-steps of 64).
-// Inputs of up to 65536 pairs and 512 experts run the same three steps inside one workgroup
-// (route_sort_single_kernel); larger ones take three launches:
+// Inputs of up to 4096 pairs and 512 experts run the same three steps inside one workgroup
+// (route_sort_single_kernel); larger ones take these steps:
 //   1. route_hist_kernel    per-chunk expert histogram in LDS (ds_add_u32), written to hist[chunk][e]
 //   2. route_scan_kernel    one wave per expert: exclusive scan of hist[:, e] over chunks (wave scan),
 //                           in place; the total is splits[e]
 //   3. route_scatter_kernel per chunk: running[e] = offsets[e] + base[chunk][e] in LDS; for each
 //                           wave-step the lanes holding the same expert are found with ballots over the
 //                           bits of the id, ranked with mbcnt, and the first of them advances running[e].
+// Up to 256 chunks (131072 pairs) step 2 is folded into step 3 (each scatter workgroup sums the histogram
+// columns it needs from L2): two launches instead of three, and launch gaps are most of the time at these sizes.
 // Every pair is read twice (8 B) and each output written once: the array traffic is the whole cost.
 #include "common.hpp"
 
@@ -20,6 +22,9 @@ constexpr int kChunk = 512;           // pairs per wave
 constexpr int kWavesPerBlock = 4;
 constexpr int kThreads = kWavesPerBlock * 64;
 constexpr int kMaxExperts = 1024;
+// Up to this many chunks (131072 pairs) the scatter kernel scans the per-chunk histograms itself (two launches);
+// beyond, a scan kernel of its own prepares them (three): the fused scan reads the table once per workgroup.
+constexpr int kFusedScanMaxChunks = 256;
 
 __global__ __launch_bounds__(kThreads) void route_hist_kernel(const int32_t *__restrict__ choosed,
                                                               int32_t npairs, int32_t nexperts,
@@ -126,24 +131,47 @@ __device__ __forceinline__ void scatter_range(const int32_t *__restrict__ choose
   }
 }
 
+// FUSED_SCAN: `base` holds the raw per-chunk histograms and every workgroup sums, per expert, the chunks ahead
+// of its own four (their starting offsets) and all chunks (the expert's total), so that the scan kernel and its
+// launch gap disappear; hist is chunks x experts int32 and sits in L2.  Used while that table is small.
+template <bool FUSED_SCAN>
 __global__ __launch_bounds__(kThreads) void route_scatter_kernel(
     const int32_t *__restrict__ choosed, int32_t npairs, int32_t topk, int32_t nexperts,
     int32_t nchunks, int32_t idbits, const int32_t *__restrict__ base,
-    const int32_t *__restrict__ splits_ws, int32_t *__restrict__ offsets_out,
+    const int32_t *__restrict__ splits_ws, int32_t *__restrict__ splits_out, int32_t *__restrict__ offsets_out,
     int32_t *__restrict__ scatter_index, int32_t *__restrict__ gather_index,
     int32_t *__restrict__ topk_index) {
-  extern __shared__ int32_t s_mem[];  // [nexperts] offsets, then [kWavesPerBlock][nexperts] running
+  extern __shared__ int32_t s_mem[];  // [nexperts] offsets, [kWavesPerBlock][nexperts] running, FUSED: [nexperts] totals
   int32_t *s_off = s_mem;
   const int wave = threadIdx.x >> 6;
   const int lane = threadIdx.x & 63;
   int32_t *running = s_mem + nexperts + wave * nexperts;
+  int32_t *s_tot = s_mem + (1 + kWavesPerBlock) * nexperts;
+  const int chunk0 = blockIdx.x * kWavesPerBlock;
+
+  if constexpr (FUSED_SCAN) {
+    for (int e = threadIdx.x; e < nexperts; e += kThreads) {
+      int sum = 0;
+      int c = 0;
+      for (; c < chunk0 && c < nchunks; ++c) sum += base[static_cast<size_t>(c) * nexperts + e];
+#pragma unroll
+      for (int w = 0; w < kWavesPerBlock; ++w, ++c) {
+        s_mem[nexperts + w * nexperts + e] = sum;  // rows of expert e in the chunks ahead of chunk0 + w
+        if (c < nchunks) sum += base[static_cast<size_t>(c) * nexperts + e];
+      }
+      for (; c < nchunks; ++c) sum += base[static_cast<size_t>(c) * nexperts + e];
+      s_tot[e] = sum;
+      if (blockIdx.x == 0 && splits_out) splits_out[e] = sum;
+    }
+    __syncthreads();
+  }
 
   // Exclusive prefix sum of splits -> offsets (every block recomputes it; E <= 1024).
   if (wave == 0) {
     int carry = 0;
     for (int e0 = 0; e0 < nexperts; e0 += 64) {
       const int e = e0 + lane;
-      const int v = e < nexperts ? splits_ws[e] : 0;
+      const int v = e < nexperts ? (FUSED_SCAN ? s_tot[e] : splits_ws[e]) : 0;
       const int incl = wave_inclusive_scan(v);
       if (e < nexperts) s_off[e] = carry + incl - v;
       carry += __shfl(incl, 63, 64);
@@ -155,10 +183,10 @@ __global__ __launch_bounds__(kThreads) void route_scatter_kernel(
   }
   __syncthreads();
 
-  const int chunk = blockIdx.x * kWavesPerBlock + wave;
+  const int chunk = chunk0 + wave;
   if (chunk >= nchunks) return;
   for (int e = lane; e < nexperts; e += 64)
-    running[e] = s_off[e] + base[static_cast<size_t>(chunk) * nexperts + e];
+    running[e] = s_off[e] + (FUSED_SCAN ? running[e] : base[static_cast<size_t>(chunk) * nexperts + e]);
   __builtin_amdgcn_wave_barrier();
 
   scatter_range<false>(choosed, nullptr, chunk * kChunk, kChunk / 64, npairs, topk, nexperts, idbits, running,
@@ -262,25 +290,16 @@ extern "C" size_t fluxmi_moe_route_sort_workspace_bytes(int32_t ntokens, int32_t
   return static_cast<size_t>((nchunks + 1) * nexperts) * sizeof(int32_t);
 }
 
-extern "C" int fluxmi_moe_route_sort(const int32_t *choosed, int32_t ntokens, int32_t topk,
-                                     int32_t nexperts, int32_t *splits, int32_t *offsets,
-                                     int32_t *scatter_index, int32_t *gather_index,
-                                     int32_t *topk_index, void *workspace, size_t workspace_bytes,
-                                     void *stream) {
-  using namespace fluxmi;
-  FLUXMI_REQUIRE(ntokens >= 0 && topk >= 1, FLUXMI_ERR_INVALID_ARG,
-                 "moe_route_sort: bad sizes (ntokens=%d, topk=%d)", ntokens, topk);
-  FLUXMI_REQUIRE(nexperts >= 1 && nexperts <= kMaxExperts, FLUXMI_ERR_UNSUPPORTED,
-                 "moe_route_sort: nexperts=%d outside [1,%d]", nexperts, kMaxExperts);
-  const int64_t npairs64 = static_cast<int64_t>(ntokens) * topk;
-  FLUXMI_REQUIRE(npairs64 <= (int64_t{1} << 30), FLUXMI_ERR_UNSUPPORTED,
-                 "moe_route_sort: ntokens*topk=%lld exceeds 2^30", static_cast<long long>(npairs64));
-  FLUXMI_REQUIRE((scatter_index != nullptr && choosed != nullptr) || npairs64 == 0,
-                 FLUXMI_ERR_INVALID_ARG, "moe_route_sort: null choosed / scatter_index");
-  const size_t need = fluxmi_moe_route_sort_workspace_bytes(ntokens, topk, nexperts);
-  FLUXMI_REQUIRE(workspace != nullptr && workspace_bytes >= need, FLUXMI_ERR_WORKSPACE,
-                 "moe_route_sort: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
-  const int32_t npairs = static_cast<int32_t>(npairs64);
+namespace fluxmi {
+namespace {
+
+// The sort itself on a workspace of at least fluxmi_moe_route_sort_workspace_bytes() bytes.  Nothing in the
+// workspace has to be zero on entry: the histogram kernel writes every hist[chunk][expert] entry (and the scan
+// kernel every splits entry) before anything reads them.
+int route_sort_on_workspace(const int32_t *choosed, int32_t ntokens, int32_t topk,
+                            int32_t nexperts, int32_t *splits, int32_t *offsets, int32_t *scatter_index,
+                            int32_t *gather_index, int32_t *topk_index, void *workspace, void *stream) {
+  const int32_t npairs = ntokens * topk;
   const int32_t nchunks = num_chunks(npairs);
   hipStream_t s = static_cast<hipStream_t>(stream);
   int32_t *splits_ws = static_cast<int32_t *>(workspace);
@@ -304,15 +323,54 @@ extern "C" int fluxmi_moe_route_sort(const int32_t *choosed, int32_t ntokens, in
                        kWavesPerBlock * nexperts * sizeof(int32_t), s, choosed, npairs, nexperts,
                        nchunks, hist);
   }
-  hipLaunchKernelGGL(route_scan_kernel, dim3((nexperts + kWavesPerBlock - 1) / kWavesPerBlock),
-                     dim3(kThreads), 0, s, hist, nexperts, nchunks, splits_ws, splits);
-  // With no pairs one block still runs to publish offsets (all zero).
-  hipLaunchKernelGGL(route_scatter_kernel, dim3(nblocks > 0 ? nblocks : 1), dim3(kThreads),
-                     (1 + kWavesPerBlock) * nexperts * sizeof(int32_t), s, choosed, npairs, topk,
-                     nexperts, nchunks, idbits, hist, splits_ws, offsets, scatter_index, gather_index,
-                     topk_index);
+  if (nchunks <= kFusedScanMaxChunks) {
+    // Two launches: every scatter workgroup scans the histogram table itself.  With no pairs one block still
+    // runs to publish splits and offsets (all zero).
+    hipLaunchKernelGGL(route_scatter_kernel<true>, dim3(nblocks > 0 ? nblocks : 1), dim3(kThreads),
+                       (2 + kWavesPerBlock) * nexperts * sizeof(int32_t), s, choosed, npairs, topk, nexperts, nchunks,
+                       idbits, hist, splits_ws, splits, offsets, scatter_index, gather_index, topk_index);
+  } else {
+    hipLaunchKernelGGL(route_scan_kernel, dim3((nexperts + kWavesPerBlock - 1) / kWavesPerBlock),
+                       dim3(kThreads), 0, s, hist, nexperts, nchunks, splits_ws, splits);
+    hipLaunchKernelGGL(route_scatter_kernel<false>, dim3(nblocks > 0 ? nblocks : 1), dim3(kThreads),
+                       (1 + kWavesPerBlock) * nexperts * sizeof(int32_t), s, choosed, npairs, topk, nexperts, nchunks,
+                       idbits, hist, splits_ws, splits, offsets, scatter_index, gather_index, topk_index);
+  }
   FLUXMI_HIP_CHECK(hipGetLastError());
   return FLUXMI_OK;
+}
+
+// Argument checks shared by the entry points.
+int route_sort_check(const char *who, const int32_t *choosed, int32_t ntokens, int32_t topk, int32_t nexperts,
+                     const int32_t *scatter_index) {
+  FLUXMI_REQUIRE(ntokens >= 0 && topk >= 1, FLUXMI_ERR_INVALID_ARG, "%s: bad sizes (ntokens=%d, topk=%d)", who,
+                 ntokens, topk);
+  FLUXMI_REQUIRE(nexperts >= 1 && nexperts <= kMaxExperts, FLUXMI_ERR_UNSUPPORTED,
+                 "%s: nexperts=%d outside [1,%d]", who, nexperts, kMaxExperts);
+  const int64_t npairs64 = static_cast<int64_t>(ntokens) * topk;
+  FLUXMI_REQUIRE(npairs64 <= (int64_t{1} << 30), FLUXMI_ERR_UNSUPPORTED, "%s: ntokens*topk=%lld exceeds 2^30", who,
+                 static_cast<long long>(npairs64));
+  FLUXMI_REQUIRE((scatter_index != nullptr && choosed != nullptr) || npairs64 == 0, FLUXMI_ERR_INVALID_ARG,
+                 "%s: null choosed / scatter_index", who);
+  return FLUXMI_OK;
+}
+
+}  // namespace
+}  // namespace fluxmi
+
+extern "C" int fluxmi_moe_route_sort(const int32_t *choosed, int32_t ntokens, int32_t topk,
+                                     int32_t nexperts, int32_t *splits, int32_t *offsets,
+                                     int32_t *scatter_index, int32_t *gather_index,
+                                     int32_t *topk_index, void *workspace, size_t workspace_bytes,
+                                     void *stream) {
+  using namespace fluxmi;
+  const int rc = route_sort_check("moe_route_sort", choosed, ntokens, topk, nexperts, scatter_index);
+  if (rc != FLUXMI_OK) return rc;
+  const size_t need = fluxmi_moe_route_sort_workspace_bytes(ntokens, topk, nexperts);
+  FLUXMI_REQUIRE(workspace != nullptr && workspace_bytes >= need, FLUXMI_ERR_WORKSPACE,
+                 "moe_route_sort: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+  return route_sort_on_workspace(choosed, ntokens, topk, nexperts, splits, offsets, scatter_index,
+                                 gather_index, topk_index, workspace, stream);
 }
 
 extern "C" int fluxmi_moe_gather_index(const int32_t *scatter_index, int32_t nrows, int32_t topk,

@@ -293,8 +293,10 @@ void GemmGroupedV3GatherRS::lazy_init(const torch::Tensor &like) {
   if (!inter_.empty()) return;
   // inter_D of the reference (gemm_grouped_v3_gather_rs.cc:165-232) is bf16; the default here is fp32 so
   // that the layer has a single rounding.  FLUX_AMD_INTER_DTYPE=bf16 restores the reference's data flow.
+  // Zero-filled once, as the reference does (init_buffer: torch::zeros): rows the GEMM never writes
+  // (sum(splits) < M) then read as zeros in the reduce instead of stale memory.
   auto opts = like.options().dtype(inter_fp32_ ? at::kFloat : at::kBFloat16);
-  for (int64_t g = 0; g < max_input_groups_; ++g) inter_.push_back(torch::empty({max_m_, n_dim_}, opts));
+  for (int64_t g = 0; g < max_input_groups_; ++g) inter_.push_back(torch::zeros({max_m_, n_dim_}, opts));
   splits_dev_ = torch::empty({num_experts_}, like.options().dtype(at::kInt));
 }
 

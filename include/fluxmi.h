@@ -84,8 +84,17 @@ int fluxmi_moe_gather_index(const int32_t *scatter_index, int32_t nrows, int32_t
  * A is row-major [*, K] (lda = K), B is [E, N, K] with K contiguous, D is row-major [*, N] bf16.
  * `splits` is a DEVICE int32 array of `nexperts` row counts; the tile schedule is derived from it on
  * the device, so the host never reads it.  `max_rows` is an upper bound of sum(splits) (ntokens*topk);
- * rows beyond sum(splits) are not touched.  Requirements: K % 64 == 0 (bf16) or K % 128 == 0 (fp8)
- * for the MFMA kernels — other K take a slower generic kernel; pointers 16-byte aligned.
+ * rows beyond sum(splits) are not touched.
+ *
+ * Limits: 1 <= nexperts <= 1024 (FLUXMI_ERR_UNSUPPORTED beyond).  Two kernels stand behind the call.  The
+ * MFMA kernel takes every shape with
+ *   - rows of K a multiple of 16 bytes: K % 8 == 0 (bf16), K % 16 == 0 (fp8); a last partial 64-byte step of
+ *     K is padded with zeros inside the kernel at full speed;
+ *   - N % 4 == 0; a, b 16-byte aligned; d 8-byte (bf16) / 16-byte (fp32) aligned; col_scale 16-byte aligned;
+ *   - one expert's weights below 4 GiB (N * K * element size), and with `gather_a`: a_rows > 0 and the whole
+ *     of A below 4 GiB (its rows are addressed with 32-bit byte offsets).
+ * Any other shape runs a generic kernel (one thread per output element, roughly 100 times slower, meant for
+ * correctness only).  fluxmi_grouped_gemm_kernel_kind() tells which of the two a call would take.
  * ---------------------------------------------------------------------------------------------- */
 typedef struct fluxmi_grouped_gemm_args {
   int32_t dtype;         /* fluxmi_dtype of A and B */
@@ -120,6 +129,12 @@ size_t fluxmi_grouped_gemm_workspace_bytes(const fluxmi_grouped_gemm_args *args)
 int fluxmi_grouped_gemm(const fluxmi_grouped_gemm_args *args, void *workspace,
                         size_t workspace_bytes, void *stream);
 
+/* Which kernel fluxmi_grouped_gemm would run for `args` (nothing is launched): 1 the MFMA kernel, 0 the
+ * generic kernel, negative = the fluxmi_status the call itself would return.  The reference has no slow
+ * path to report (its TMA kernels take any 16-byte aligned K: gemm_grouped_v3_ag_scatter.cc:249-262 checks
+ * shapes only); callers use this to assert they are not on the generic kernel. */
+int fluxmi_grouped_gemm_kernel_kind(const fluxmi_grouped_gemm_args *args);
+
 /* The same rows times `ngroups` (1..4) weight tensors in ONE launch, each group with an output of its own:
  * `GemmGroupedV3AGScatterOp::forward_multiple_weights` (gate and up projections sharing the gathered
  * A tiles; src/moe_ag_scatter/ths_op/gemm_grouped_v3_ag_scatter.cc:375-395).  b, d and alpha are
@@ -140,10 +155,12 @@ int fluxmi_grouped_gemm_multi(const fluxmi_grouped_gemm_args *args, int32_t ngro
  *
  *   out[t, n] = bf16( scale * sum_{g < ngroups} sum_{j < topk}
  *                       w[r] * float(in[g][r, n]) ),   r = routing_idx[t*topk + j],
- *   w[r] = row_weight ? row_weight[r] : 1;  rows with r < 0 are skipped; fp32 accumulation in the
- *   order g-major then j; one rounding at the end.
- * `in` is an array (on the HOST) of `ngroups` device pointers to row-major [nrows, n] matrices, bf16, or
- * fp32 when `in_fp32` != 0 (the unrounded intermediate of fluxmi_grouped_gemm with d_fp32 = 1).
+ *   w[r] = row_weight ? row_weight[r] : 1;  fp32 accumulation in the order g-major then j; one rounding at
+ *   the end.
+ * `in` is an array (on the HOST) of `ngroups` device pointers to row-major [ntokens*topk, n] matrices, bf16,
+ * or fp32 when `in_fp32` != 0 (the unrounded intermediate of fluxmi_grouped_gemm with d_fp32 = 1).  Entries of
+ * routing_idx outside [0, ntokens*topk) name no row: they are skipped (negative = a dropped pair) and never
+ * dereferenced.
  * Requirements: n % 8 == 0, 1 <= ngroups <= 4, 1 <= topk <= 64.
  * ---------------------------------------------------------------------------------------------- */
 int fluxmi_topk_gather_reduce(const void *const *in, int32_t ngroups, int32_t in_fp32,

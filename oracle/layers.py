@@ -89,8 +89,10 @@ def layer1_fp32(a_sorted, weights, split, routing_idx, topk, input_scale=None, w
 def layer1_torch(a_sorted, weights, split, gather_idx, topk_idx, topk, input_scale=None, weight_scale=None,
                  output_vec_scale=None):
     """moe_gather_rs_forward_torch at world size 1 (python/flux/testing/moe_gather_rs_utils.py:26-120):
-    per expert scale_v * matmul (:89), concat, times output_vec_scale and round to bf16 (:95), scatter to
-    row topk*token_index + topk_index (:96-102), view(T, topk, N).sum(1) (:104)."""
+    per expert scale_v * matmul (:89; a python float times a bf16 tensor stays bf16, so the product is
+    rounded), concat, times output_vec_scale and round to bf16 (:95), scatter to row
+    topk*token_index + topk_index (:96-102), view(T, topk, N).sum(1) (:104).  Three roundings before the
+    sum: the matmul result, the scaled result, the weighted result."""
     dt = a_sorted.dtype
     m, n = a_sorted.shape[0], weights.shape[1]
     off = routing.offsets(np.asarray(split))
@@ -100,10 +102,10 @@ def layer1_torch(a_sorted, weights, split, gather_idx, topk_idx, topk, input_sca
         lo, hi = int(off[e]), int(off[e + 1])
         s_w = 1.0 if weight_scale is None else float(weight_scale[e])
         y = (_f32(a_sorted[lo:hi]) @ _f32(weights[e]).t()).to(dt)  # torch.matmul in bf16
-        parts.append((s_w * s_in) * _f32(y))
-    out = torch.cat(parts) if parts else torch.zeros(0, n)
+        parts.append(((s_w * s_in) * _f32(y)).to(dt))          # scale_v * bf16 tensor -> bf16
+    out = _f32(torch.cat(parts)) if parts else torch.zeros(0, n)
     if output_vec_scale is not None:
-        out = out * output_vec_scale.to(torch.float32)[:, None]
+        out = out * output_vec_scale.to(torch.float32)[:, None]  # bf16 * fp32 tensor -> fp32
     out = out.to(dt)
     new_index = topk * torch.as_tensor(np.asarray(gather_idx), dtype=torch.long) + torch.as_tensor(
         np.asarray(topk_idx), dtype=torch.long)

@@ -107,3 +107,28 @@ def test_benchmark_shapes_properties(name):
     tot_in = inter.float().sum(0).cpu()
     tot_out = ones.float().sum(0).cpu()
     assert torch.allclose(tot_in, tot_out, rtol=2e-2, atol=float(m) ** 0.5 * 0.05)
+
+
+@pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("topk", [2, 3])
+def test_routing_entries_outside_the_input_are_skipped(in_dtype, topk):
+    """An entry of routing_idx at or beyond ntokens*topk names no row: it must contribute nothing and must not be
+    dereferenced (the input is followed by NaNs here; entries point far past it as well)."""
+    from flux_amd import capi
+    g = torch.Generator().manual_seed(9)
+    tokens, n = 64, 512
+    m = tokens * topk
+    buf = torch.full((m + 8, n), float("nan"), dtype=in_dtype)
+    inter = torch.randn(m, n, generator=g).to(in_dtype)
+    buf[:m] = inter
+    idx = torch.randperm(m, generator=g).to(torch.int32)
+    bad = idx.clone()
+    bad[3], bad[10], bad[77] = m, m + 5, 2 ** 31 - 1
+    w = torch.rand(m, generator=g) + 0.5
+    ref_idx = bad.clone()
+    ref_idx[ref_idx >= m] = -1
+    ref = layers.topk_gather_reduce_fp32(inter, ref_idx.numpy(), topk, row_weight=w)
+    out = capi.topk_gather_reduce(buf.cuda()[:m], bad.cuda(), topk, row_weight=w.cuda())
+    got = out.float().cpu()
+    assert not bool(torch.isnan(got).any())
+    assert torch.allclose(got, ref, rtol=1e-2, atol=1e-2)

@@ -194,6 +194,61 @@ def test_fp8_layer1_through_ops():
     assert err < 3e-2, err
 
 
+def test_fp8_c5_chain_through_ops_full_size():
+    """C5 at full size through the operator classes, the reference's call sequence (examples/moe_flux_only.py:112-131):
+    layer0 GemmGroupedV3AGScatter on e4m3 tokens and weights with the reference's fp8 scale form (one activation
+    scale, one scale per expert, folded into output_scale [E]; python/flux/cpp_mod.pyi:932-938), its bf16 output
+    quantised per row, layer1 GemmGroupedV3GatherRS with input_scale [M] x weight_scale [E, N] and the top-8
+    weights as output_vec_scale.  Sampled rows / tokens against the dequantise-matmul oracle on the same bytes."""
+    wl = configs.make_workload("C5")
+    t, k, e, h, f, m = wl.tokens, wl.topk, wl.experts, wl.hidden, wl.ffn, wl.rows
+    print(f"[case] ops chain fp8 C5 T={t} k={k} E={e} H={h} F={f}", flush=True)
+    rng = np.random.default_rng(73)
+    q = flux_amd.Quantization(torch.bfloat16, torch.float8_e4m3fn)
+    x, w1, w2 = (wl.tensors[n].cuda() for n in ("x", "w1", "w2"))
+    # layer0 operands: per-tensor activation scale, per-expert weight scale
+    sx = float(x.float().abs().max()) / 448.0
+    qx = (x.float() / sx).to(torch.float8_e4m3fn)
+    sw1 = w1.float().abs().amax(dim=(1, 2)) / 448.0
+    qw1 = (w1.float() / sw1[:, None, None]).to(torch.float8_e4m3fn)
+    output_scale = (sw1 * sx).contiguous()
+    splits_gpu = torch.from_numpy(wl.splits).cuda()
+    scatter_index = torch.from_numpy(wl.scatter_index).cuda()
+    op0 = flux_amd.GemmGroupedV3AGScatter(flux_amd.DistEnvTPWithEP(None, 1, None),
+                                          flux_amd.MoeArguments(t, h, f, e, k, torch.float8_e4m3fn, torch.bfloat16))
+    y = op0.forward(qx, qw1, splits_gpu, scatter_index, output_scale=output_scale, fast_accum=False)
+    assert y.dtype == torch.bfloat16 and tuple(y.shape) == (m, f)
+    eor = routing.expert_of_row(wl.splits)
+    off = routing.offsets(wl.splits)
+    rows = np.concatenate([np.array([off[i], off[i + 1] - 1]) for i in range(e) if off[i + 1] > off[i]]
+                          + [rng.integers(0, m, size=64)])
+    qx_c, qw1_c, os_c = qx.cpu().float(), qw1.cpu(), output_scale.cpu()
+    for r in rows:
+        ee = int(eor[r])
+        ref = (qx_c[int(wl.gather_index[r])] @ qw1_c[ee].float().t()) * float(os_c[ee])
+        got = y[int(r)].float().cpu()
+        assert torch.allclose(got, ref, rtol=1e-2, atol=1e-2 * float(ref.abs().max())), f"layer0 row {r}"
+    # layer1: per-row activation scales, per-output-channel weight scales
+    qa, sa = q.quantize_rowwise(y)
+    qw2, sw2 = q.quantize_rowwise(w2.reshape(-1, f))
+    qw2, sw2 = qw2.reshape(e, h, f), sw2.reshape(e, h)
+    op1 = flux_amd.GemmGroupedV3GatherRS(e, m, h, k, 0, 1, 1, 1)
+    out = op1.forward_gather_rs(qa, qw2, torch.from_numpy(wl.splits), scatter_index.view(-1), input_scale=sa,
+                                weight_scale=sw2, output_vec_scale=wl.row_weight.cuda(), fast_accum=False)
+    assert out.dtype == torch.bfloat16 and tuple(out.shape) == (t, h)
+    qa_c, sa_c, qw2_c, sw2_c = qa.cpu(), sa.cpu(), qw2.cpu(), sw2.cpu()
+    tok = rng.integers(0, t, size=12)
+    ref1 = torch.zeros(len(tok), h)
+    for i, tt in enumerate(tok):
+        for j in range(k):
+            r = int(wl.scatter_index[tt, j])
+            ee = int(eor[r])
+            ref1[i] += float(wl.row_weight[r]) * float(sa_c[r]) * ((qa_c[r].float() @ qw2_c[ee].float().t()) * sw2_c[ee])
+    got = out[torch.as_tensor(tok).cuda()].float().cpu()
+    assert float((got - ref1).norm() / ref1.norm()) < 3e-2
+    assert torch.allclose(got, ref1, rtol=1e-2, atol=1e-2 * float(ref1.abs().max()))
+
+
 def test_profiling_registers_a_schedule_and_keeps_results(c1):
     """profiling() of both layer ops: every tile schedule gives the bits of forward(); the fastest is recorded in
     the context, registered for the shape, and its text form loads back."""

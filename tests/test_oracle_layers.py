@@ -103,6 +103,21 @@ def test_layer1_forms_agree():
     assert torch.allclose(a.double(), ref, rtol=1e-5, atol=1e-6)
 
 
+def test_layer1_torch_rounds_after_the_scalar_scale():
+    """scale_v * torch.matmul(...) of the reference (python/flux/testing/moe_gather_rs_utils.py:89) is a python
+    float times a bf16 tensor, i.e. bf16: the scaled product is rounded before output_vec_scale is applied.
+    Hand-computed case that tells the two forms apart: y = 1.0078125 (bf16), scale_v = 1 + 2^-8, weight 0.998:
+      three roundings: bf16(1.0117797...) = 1.015625 (above the midpoint 1.01171875), times 0.998 = 1.01359 -> 1.015625
+      without the middle rounding: 1.0117797 * 0.998 = 1.009756 -> 1.0078125."""
+    act = torch.tensor([[1.0]], dtype=torch.bfloat16)
+    w = torch.tensor([[[1.0078125]]], dtype=torch.bfloat16)
+    split = np.array([1], dtype=np.int32)
+    gi, ti = np.array([0]), np.array([0])
+    out = layers.layer1_torch(act, w, split, gi, ti, 1, None, torch.tensor([1.00390625]), torch.tensor([0.998]))
+    assert out.dtype == torch.bfloat16 and float(out[0, 0]) == 1.015625
+    assert float(torch.tensor(1.0078125 * 1.00390625 * 0.998).to(torch.bfloat16)) == 1.0078125  # the two-rounding value
+
+
 def test_reference_debug_closed_form():
     """The --debug data of test/python/moe_gather_rs/test_moe_gather_rs.py:502-518: x[:,0] = (i+1) % M, rest 0,
     W = 1, output_vec_scale = 2  =>  every output column of token t equals 2 * sum_j x[row_j, 0]."""
