@@ -18,6 +18,7 @@ FP8_E4M3 = 1
 EXPORTS = (
     "fluxmi_version", "fluxmi_last_error", "fluxmi_device_cu_count",
     "fluxmi_moe_route_sort_workspace_bytes", "fluxmi_moe_route_sort", "fluxmi_moe_gather_index",
+    "fluxmi_moe_route_sort_static_max_bytes", "fluxmi_moe_route_sort_static",
     "fluxmi_grouped_gemm_workspace_bytes", "fluxmi_grouped_gemm", "fluxmi_grouped_gemm_kernel_kind",
     "fluxmi_grouped_gemm_multi",
     "fluxmi_topk_gather_reduce", "fluxmi_quant_e4m3_rowwise", "fluxmi_quant_e4m3_square",
@@ -60,6 +61,8 @@ def load():
     lib.fluxmi_moe_route_sort_workspace_bytes.argtypes = [i32, i32, i32]
     lib.fluxmi_moe_route_sort.argtypes = [vp, i32, i32, i32, vp, vp, vp, vp, vp, vp, sz, vp]
     lib.fluxmi_moe_gather_index.argtypes = [vp, i32, i32, vp, vp, vp]
+    lib.fluxmi_moe_route_sort_static_max_bytes.restype = sz
+    lib.fluxmi_moe_route_sort_static.argtypes = [vp, i32, i32, i32, vp, vp, vp, vp, vp, vp]
     lib.fluxmi_grouped_gemm_workspace_bytes.restype = sz
     lib.fluxmi_grouped_gemm_workspace_bytes.argtypes = [ctypes.POINTER(GroupedGemmArgs)]
     lib.fluxmi_grouped_gemm.argtypes = [ctypes.POINTER(GroupedGemmArgs), vp, sz, vp]
@@ -111,6 +114,22 @@ def route_sort(choosed, nexperts, want_gather=True, want_topk_index=True):
                                      _ptr(scatter), _ptr(gather), _ptr(tki), _ptr(ws), ws_bytes, _stream()),
            "fluxmi_moe_route_sort")
     return splits, offsets, scatter, gather, tki
+
+
+def route_sort_static(choosed, nexperts, out):
+    """fluxmi_moe_route_sort_static into the caller's tensors `out` = (splits, offsets, scatter_index,
+    gather_index, topk_index), the last two optional (None).  Allocates nothing, here or in the library."""
+    lib = load()
+    _dev_tensor(choosed, torch.int32, "choosed")
+    ntokens, topk = choosed.shape
+    splits, offsets, scatter, gather, tki = out
+    for nm, t in (("splits", splits), ("offsets", offsets), ("scatter_index", scatter), ("gather_index", gather),
+                  ("topk_index", tki)):
+        _dev_tensor(t, torch.int32, nm)
+    _check(lib.fluxmi_moe_route_sort_static(_ptr(choosed), ntokens, topk, nexperts, _ptr(splits), _ptr(offsets),
+                                            _ptr(scatter), _ptr(gather), _ptr(tki), _stream()),
+           "fluxmi_moe_route_sort_static")
+    return out
 
 
 def gather_index(scatter_index, topk):

@@ -373,6 +373,56 @@ extern "C" int fluxmi_moe_route_sort(const int32_t *choosed, int32_t ntokens, in
                                  gather_index, topk_index, workspace, stream);
 }
 
+// ---- entry point that allocates nothing --------------------------------------------------------------------
+// The sort's scratch (per-chunk histograms) in a file-scope device array instead of a caller's workspace, for
+// callers that cannot allocate.  Every GPU holds its own copy of the array at its own address; the address is
+// looked up once per device and kept.  In host code the array's name is only a handle for that lookup.
+namespace fluxmi {
+namespace {
+
+constexpr size_t kStaticScratchBytes = size_t{4} << 20;  // 4 MiB per GPU, held until the process ends
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+std::atomic<void *> g_scratch_ptr[64];  // device id -> device address of `scratch` on that GPU
+
+int static_scratch(void **out) {
+  int dev = 0;
+  FLUXMI_HIP_CHECK(hipGetDevice(&dev));
+  FLUXMI_REQUIRE(dev >= 0 && dev < 64, FLUXMI_ERR_UNSUPPORTED, "moe_route_sort_static: device id %d outside [0,64)", dev);
+  void *ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (ptr == nullptr) {
+    FLUXMI_HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    FLUXMI_REQUIRE(ptr != nullptr, FLUXMI_ERR_HIP, "moe_route_sort_static: no device address for the scratch array");
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);  // a lost race stores the same address
+  }
+  *out = ptr;
+  return FLUXMI_OK;
+}
+
+}  // namespace
+}  // namespace fluxmi
+
+extern "C" size_t fluxmi_moe_route_sort_static_max_bytes(void) { return fluxmi::kStaticScratchBytes; }
+
+extern "C" int fluxmi_moe_route_sort_static(const int32_t *choosed, int32_t ntokens, int32_t topk,
+                                            int32_t nexperts, int32_t *splits, int32_t *offsets,
+                                            int32_t *scatter_index, int32_t *gather_index,
+                                            int32_t *topk_index, void *stream) {
+  using namespace fluxmi;
+  const int rc = route_sort_check("moe_route_sort_static", choosed, ntokens, topk, nexperts, scatter_index);
+  if (rc != FLUXMI_OK) return rc;
+  const size_t need = fluxmi_moe_route_sort_workspace_bytes(ntokens, topk, nexperts);
+  FLUXMI_REQUIRE(need <= kStaticScratchBytes, FLUXMI_ERR_WORKSPACE,
+                 "moe_route_sort_static: ntokens=%d topk=%d nexperts=%d needs %zu bytes of scratch, the static "
+                 "array holds %zu; use fluxmi_moe_route_sort with a workspace",
+                 ntokens, topk, nexperts, need, kStaticScratchBytes);
+  void *ws = nullptr;
+  const int rs = static_scratch(&ws);
+  if (rs != FLUXMI_OK) return rs;
+  return route_sort_on_workspace(choosed, ntokens, topk, nexperts, splits, offsets, scatter_index, gather_index,
+                                 topk_index, ws, stream);
+}
+
 extern "C" int fluxmi_moe_gather_index(const int32_t *scatter_index, int32_t nrows, int32_t topk,
                                        int32_t *gather_index, int32_t *topk_index, void *stream) {
   using namespace fluxmi;

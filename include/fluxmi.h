@@ -60,6 +60,19 @@ int fluxmi_moe_route_sort(const int32_t *choosed, int32_t ntokens, int32_t topk,
                           int32_t *gather_index, int32_t *topk_index, void *workspace,
                           size_t workspace_bytes, void *stream);
 
+/* The same sort for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The scratch the sort needs lives
+ * in a device array inside the library (fluxmi_moe_route_sort_static_max_bytes() = 4 MiB per GPU, held until
+ * the process ends); the call itself allocates and frees nothing.  Inputs whose
+ * fluxmi_moe_route_sort_workspace_bytes() exceeds that size are rejected with FLUXMI_ERR_WORKSPACE (the limit
+ * is (ceil(ntokens*topk / 512) + 1) * nexperts <= 1048576).  All calls on one GPU share the one array: calls
+ * that overlap in time on the same GPU (different streams or threads) race; calls on one stream are ordered.
+ * Results are bit-identical to fluxmi_moe_route_sort. */
+size_t fluxmi_moe_route_sort_static_max_bytes(void);
+int fluxmi_moe_route_sort_static(const int32_t *choosed, int32_t ntokens, int32_t topk, int32_t nexperts,
+                                 int32_t *splits, int32_t *offsets, int32_t *scatter_index,
+                                 int32_t *gather_index, int32_t *topk_index, void *stream);
+
 /* Inverse permutation only: `calc_gather_index_impl` (src/moe_ag_scatter/sort_util.cu:121-160).
  * gather_index[scatter_index[i]] = i / topk, topk_index[...] = i % topk for scatter_index[i] in
  * [0, nrows); entries outside are skipped.  topk_index may be NULL. */
