@@ -29,7 +29,7 @@ def _load_ths():
 
 _THS_NAMES = (
     "MoeArguments", "DistEnvTPWithEP", "GemmGroupedV3AGScatter", "GemmGroupedV3GatherRS", "GemmGroupedV3",
-    "Quantization", "calc_scatter_index", "topk_scatter_reduce", "bitwise_check", "init_flux_shm",
+    "Quantization", "BlockScaleGemm", "calc_scatter_index", "topk_scatter_reduce", "bitwise_check", "init_flux_shm",
     "moe_route_sort", "topk_weighted_gather_reduce", "uniform_initialize", "load_tuning_record",
     "ProfilingContext", "TuningRecord", "load_tuning_text",
 )

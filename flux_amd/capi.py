@@ -20,7 +20,8 @@ EXPORTS = (
     "fluxmi_moe_route_sort_workspace_bytes", "fluxmi_moe_route_sort", "fluxmi_moe_gather_index",
     "fluxmi_moe_route_sort_static_max_bytes", "fluxmi_moe_route_sort_static",
     "fluxmi_grouped_gemm_workspace_bytes", "fluxmi_grouped_gemm", "fluxmi_grouped_gemm_kernel_kind",
-    "fluxmi_grouped_gemm_multi",
+    "fluxmi_grouped_gemm_multi", "fluxmi_grouped_gemm_topk_reduce_workspace_bytes",
+    "fluxmi_grouped_gemm_topk_reduce", "fluxmi_grouped_gemm_blockscale",
     "fluxmi_topk_gather_reduce", "fluxmi_quant_e4m3_rowwise", "fluxmi_quant_e4m3_square",
     "fluxmi_quant_e4m3_block128",
 )
@@ -67,6 +68,10 @@ def load():
     lib.fluxmi_grouped_gemm_workspace_bytes.argtypes = [ctypes.POINTER(GroupedGemmArgs)]
     lib.fluxmi_grouped_gemm.argtypes = [ctypes.POINTER(GroupedGemmArgs), vp, sz, vp]
     lib.fluxmi_grouped_gemm_kernel_kind.argtypes = [ctypes.POINTER(GroupedGemmArgs)]
+    lib.fluxmi_grouped_gemm_topk_reduce_workspace_bytes.restype = sz
+    lib.fluxmi_grouped_gemm_topk_reduce_workspace_bytes.argtypes = [i32, i32]
+    lib.fluxmi_grouped_gemm_topk_reduce.argtypes = [ctypes.POINTER(GroupedGemmArgs), vp, i32, vp, vp, sz, vp]
+    lib.fluxmi_grouped_gemm_blockscale.argtypes = [ctypes.POINTER(GroupedGemmArgs), vp, i32, vp, i32, vp]
     lib.fluxmi_grouped_gemm_multi.argtypes = [ctypes.POINTER(GroupedGemmArgs), i32, vp, vp, vp, vp, sz, vp]
     lib.fluxmi_topk_gather_reduce.argtypes = [ctypes.POINTER(vp), i32, i32, vp, vp, f32, i32, i32, i32, vp, vp]
     lib.fluxmi_quant_e4m3_rowwise.argtypes = [vp, i64, i64, i32, f32, vp, vp, i32, vp]
@@ -147,12 +152,8 @@ SCHED_WHOLE_TAIL_TILES = 1
 SCHED_NO_HALF_TILES = 2
 
 
-def grouped_gemm(a, b, splits, out=None, gather_a=None, scatter_d=None, alpha=None, row_scale=None,
-                 col_scale=None, scalar_scale=1.0, scalar_scale_dev=None, max_rows=None, out_dtype=None,
-                 cu_margin=0, raster_rows=0, sched_flags=0, want_kind=False):
-    """D = grouped GEMM of A [rows_a, K] with B [E, N, K]; see fluxmi_grouped_gemm in include/fluxmi.h.
-    With `want_kind` the result is (D, kind): kind 1 = the MFMA kernel ran, 0 = the generic kernel."""
-    lib = load()
+def _gemm_args(a, b, splits, out, gather_a, scatter_d, alpha, row_scale, col_scale, scalar_scale, scalar_scale_dev,
+               max_rows, out_dtype, cu_margin, raster_rows, sched_flags, need_out=True):
     if a.dtype == torch.bfloat16:
         dtype = BF16
     elif a.dtype == torch.float8_e4m3fn:
@@ -172,27 +173,79 @@ def grouped_gemm(a, b, splits, out=None, gather_a=None, scatter_d=None, alpha=No
         raise ValueError(f"K mismatch: a {tuple(a.shape)} vs b {tuple(b.shape)}")
     if max_rows is None:
         max_rows = gather_a.numel() if gather_a is not None else a.shape[0]
-    if out is None:
-        out = torch.empty(max_rows, n, dtype=out_dtype or torch.bfloat16, device=a.device)
-    if out.dtype not in (torch.bfloat16, torch.float32):
-        raise ValueError(f"out must be bf16 or fp32, got {out.dtype}")
-    _dev_tensor(out, out.dtype, "out")
-    if out.shape[0] < max_rows or out.shape[1] != n:
-        raise ValueError(f"out {tuple(out.shape)} too small for [{max_rows}, {n}]")
+    if need_out:
+        if out is None:
+            out = torch.empty(max_rows, n, dtype=out_dtype or torch.bfloat16, device=a.device)
+        if out.dtype not in (torch.bfloat16, torch.float32):
+            raise ValueError(f"out must be bf16 or fp32, got {out.dtype}")
+        _dev_tensor(out, out.dtype, "out")
+        if out.shape[0] < max_rows or out.shape[1] != n:
+            raise ValueError(f"out {tuple(out.shape)} too small for [{max_rows}, {n}]")
     args = GroupedGemmArgs(
         dtype=dtype, nexperts=e, max_rows=max_rows, n=n, k=k, a_rows=a.shape[0],
-        a=a.data_ptr(), b=b.data_ptr(), d=out.data_ptr(), splits=splits.data_ptr(),
+        a=a.data_ptr(), b=b.data_ptr(), d=out.data_ptr() if need_out else None, splits=splits.data_ptr(),
         gather_a=None if gather_a is None else gather_a.data_ptr(),
         scatter_d=None if scatter_d is None else scatter_d.data_ptr(),
         alpha=None if alpha is None else alpha.data_ptr(),
         row_scale=None if row_scale is None else row_scale.data_ptr(),
         col_scale=None if col_scale is None else col_scale.data_ptr(),
-        scalar_scale=float(scalar_scale), d_fp32=int(out.dtype == torch.float32),
+        scalar_scale=float(scalar_scale), d_fp32=int(need_out and out.dtype == torch.float32),
         scalar_scale_dev=None if scalar_scale_dev is None else scalar_scale_dev.data_ptr(),
         cu_margin=cu_margin, raster_rows=raster_rows, sched_flags=sched_flags)
+    return args, out
+
+
+def grouped_gemm(a, b, splits, out=None, gather_a=None, scatter_d=None, alpha=None, row_scale=None,
+                 col_scale=None, scalar_scale=1.0, scalar_scale_dev=None, max_rows=None, out_dtype=None,
+                 cu_margin=0, raster_rows=0, sched_flags=0, want_kind=False):
+    """D = grouped GEMM of A [rows_a, K] with B [E, N, K]; see fluxmi_grouped_gemm in include/fluxmi.h.
+    With `want_kind` the result is (D, kind): kind 1 = the MFMA kernel ran, 0 = the generic kernel."""
+    lib = load()
+    args, out = _gemm_args(a, b, splits, out, gather_a, scatter_d, alpha, row_scale, col_scale, scalar_scale,
+                           scalar_scale_dev, max_rows, out_dtype, cu_margin, raster_rows, sched_flags)
     _check(lib.fluxmi_grouped_gemm(ctypes.byref(args), None, 0, _stream()), "fluxmi_grouped_gemm")
     if want_kind:
         return out, lib.fluxmi_grouped_gemm_kernel_kind(ctypes.byref(args))
+    return out
+
+
+ASCALE_BLOCK128, ASCALE_EXPERT_K_M = 0, 1
+BSCALE_N_K, BSCALE_K_N = 0, 1
+
+
+def grouped_gemm_blockscale(a, b, splits, a_scale, b_scale, a_scale_layout=ASCALE_BLOCK128, b_scale_layout=BSCALE_N_K,
+                            out=None, gather_a=None, scatter_d=None, alpha=None, row_scale=None, col_scale=None,
+                            scalar_scale=1.0, max_rows=None, out_dtype=None):
+    """Block-scaled fp8 grouped GEMM (fluxmi_grouped_gemm_blockscale): a_scale per (row of A, 128 of K), b_scale
+    per 128 x 128 block of each B[e]; layouts as in include/fluxmi.h."""
+    lib = load()
+    _dev_tensor(a_scale, torch.float32, "a_scale")
+    _dev_tensor(b_scale, torch.float32, "b_scale")
+    args, out = _gemm_args(a, b, splits, out, gather_a, scatter_d, alpha, row_scale, col_scale, scalar_scale, None,
+                           max_rows, out_dtype, 0, 0, 0)
+    _check(lib.fluxmi_grouped_gemm_blockscale(ctypes.byref(args), _ptr(a_scale), a_scale_layout, _ptr(b_scale),
+                                              b_scale_layout, _stream()), "fluxmi_grouped_gemm_blockscale")
+    return out
+
+
+def grouped_gemm_topk_reduce(a, b, splits, token_of_row, ntokens, out=None, workspace=None, gather_a=None, alpha=None,
+                             row_scale=None, col_scale=None, scalar_scale=1.0, scalar_scale_dev=None, max_rows=None):
+    """out[t] = bf16(sum of the scaled GEMM rows r with token_of_row[r] == t): the top-k reduction fused into the
+    grouped GEMM's epilogue (fluxmi_grouped_gemm_topk_reduce).  `workspace`: fp32 [ntokens, N] scratch."""
+    lib = load()
+    _dev_tensor(token_of_row, torch.int32, "token_of_row")
+    args, _ = _gemm_args(a, b, splits, None, gather_a, None, alpha, row_scale, col_scale, scalar_scale,
+                         scalar_scale_dev, max_rows, None, 0, 0, 0, need_out=False)
+    n = b.shape[1]
+    if out is None:
+        out = torch.empty(ntokens, n, dtype=torch.bfloat16, device=a.device)
+    _dev_tensor(out, torch.bfloat16, "out")
+    ws_bytes = lib.fluxmi_grouped_gemm_topk_reduce_workspace_bytes(ntokens, n)
+    if workspace is None:
+        workspace = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=a.device)
+    _check(lib.fluxmi_grouped_gemm_topk_reduce(ctypes.byref(args), _ptr(token_of_row), ntokens, _ptr(out),
+                                               _ptr(workspace), workspace.numel() * workspace.element_size(), _stream()),
+           "fluxmi_grouped_gemm_topk_reduce")
     return out
 
 

@@ -83,11 +83,19 @@ struct GemmParams {
   int32_t raster_rows;  // row tiles per raster group, >= 1
   int32_t sched_flags;  // FLUXMI_SCHED_*
   int32_t nt_stores;    // fp32 outputs are stored non-temporally
+  int32_t accumulate;   // D is fp32 and every result is added to it atomically (rows meeting in one D row sum up)
+  int32_t d_rows;       // rows of D: bound for scatter_d entries
+  // Block-scaled fp8 (one scale per row of A and 128 of K, one per 128 x 128 block of B); null otherwise.
+  const float *a_scale;
+  const float *b_scale;
+  int32_t a_scale_layout;  // FLUXMI_ASCALE_*
+  int32_t b_scale_layout;  // FLUXMI_BSCALE_*
 };
 
 
 // One launcher per element type, each in a translation unit of its own (the kernel is a long compile).
 int launch_grouped_gemm_bf16(const GemmParams &p, int grid, hipStream_t s);
 int launch_grouped_gemm_fp8(const GemmParams &p, int grid, hipStream_t s);
+int launch_grouped_gemm_fp8_blockscale(const GemmParams &p, int grid, hipStream_t s);
 
 }  // namespace fluxmi

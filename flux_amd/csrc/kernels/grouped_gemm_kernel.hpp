@@ -141,8 +141,9 @@ __device__ __forceinline__ void store_tile(uint8_t *windows, const TileCtx &c, i
   uint8_t *dlane = d + (static_cast<int64_t>(row_base + wrow0 + rr0) * n + wcol0 + cc * 4) * ELT_OUT;
   const int64_t rowgroup_bytes = static_cast<int64_t>(8) * n * ELT_OUT;
   const int32_t *scatter = FULL ? nullptr : p->scatter_d;
-  const int max_rows = p->max_rows;
+  const int d_rows = p->d_rows;
   const bool nt_stores = p->nt_stores != 0;  // wave-uniform
+  const bool accumulate = !FULL && p->accumulate != 0;
   if constexpr (ELT == 2 && !OUT_F32 && FULL && NB % 2 == 0) {
     // bf16 rows of whole tiles leave as whole 128-byte lines: two 32-column blocks per pass, packed to bf16
     // before the pass, so that the window (64 rows x 128 bytes) comes back as eight lanes x 16 bytes per row.
@@ -238,14 +239,21 @@ __device__ __forceinline__ void store_tile(uint8_t *windows, const TileCtx &c, i
           if (m >= rows_e || col >= n) continue;  // n % 4 == 0: a chunk is all in or all out
           if (scatter) {
             const int64_t drow = scatter[row_base + m];
-            if (drow < 0 || drow >= max_rows) continue;
+            if (drow < 0 || drow >= d_rows) continue;
             dst = d + (drow * n + col) * ELT_OUT;
           }
         }
         float4 o = v[it];
         if constexpr (SCALED) o = make_float4(o.x * cs.x, o.y * cs.y, o.z * cs.z, o.w * cs.w);
         if constexpr (OUT_F32) {
-          if (nt_stores) {
+          if (accumulate) {
+            // Hardware fp32 atomic adds without return: sorted rows of one token meet in that token's row of D.
+            float *df = reinterpret_cast<float *>(dst);
+            unsafeAtomicAdd(df + 0, o.x);
+            unsafeAtomicAdd(df + 1, o.y);
+            unsafeAtomicAdd(df + 2, o.z);
+            unsafeAtomicAdd(df + 3, o.w);
+          } else if (nt_stores) {
             typedef float f32x4_t __attribute__((ext_vector_type(4)));
             const f32x4_t ov = {o.x, o.y, o.z, o.w};
             __builtin_nontemporal_store(ov, reinterpret_cast<f32x4_t *>(dst));
@@ -416,9 +424,16 @@ __device__ __forceinline__ void issue_first_pairs(const TileOperands<XL, WL> &op
 // (MB, NB) = (4, 4) is the macro tile, (2, 4) its upper half (for the last rows of an expert); (4, 2) and
 // (2, 2) are the 256x128 and 128x128 pieces a tile of the last, partly filled round is cut into.  Waves
 // are laid out 2 x 2.
-template <int ELT, int MB, int NB>
+//
+// BS (block-scaled fp8, 256 x 128 tiles only): A carries one scale per row and 128 of K, B one per 128 x 128
+// block.  A pair of k-steps is one scale block of K: its products are summed in `acc`, and at the end of the
+// pair main += acc * a_scale[row] * b_scale, acc = 0.  The 256 row scales of a pair travel like its operands: one
+// more direct-to-LDS fill per wave (64 rows x 4 bytes), the first instruction of the pair's fills, into the
+// half of the pair's first ring stage that a 128-column W tile leaves unused; the wait counts below include it.
+template <int ELT, int MB, int NB, bool BS = false>
 __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, const TileCtx &c, const TileDesc &t,
                                           const TileDesc &next, TilePrefetch &pf) {
+  static_assert(!BS || (ELT == 1 && MB == 4 && NB == 2), "block scales: fp8, 256 x 128 tiles");
   constexpr int XLOADS = MB;           // direct-to-LDS instructions per wave per stage, X tile
   constexpr int WLOADS = NB;           // same, W tile
   constexpr int LOADS = XLOADS + WLOADS;
@@ -428,6 +443,11 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
   constexpr int NR = (MBK + NBK) * NCH;  // fragment reads per k-step (16 bytes per lane each)
   constexpr int NM = MBK * NBK;          // MFMAs per k-step
   constexpr int RSPAN = NM / 2;        // MFMA slots over which the fragment reads of a step are spread
+  constexpr int PAIR = 2 * LOADS + (BS ? 1 : 0);  // vector-memory instructions per wave and pair of k-steps
+  constexpr int HALF = LOADS + (BS ? 1 : 0);      // ... of which the pair's first step issues this many
+  constexpr int WAIT_EVEN = (LA - 2) / 2 * PAIR;  // outstanding fills allowed when an even step starts
+  constexpr int WAIT_ODD = (LA - 4) / 2 * PAIR + HALF;
+  constexpr int SCALE_OFF = XB + W_TILE_BYTES / 2;  // row scales of a pair inside its first stage (BS)
   const int wave = c.wave, lane = c.lane, wm = c.wm, wn = c.wn, nk = c.nk;
   const int e = t.e, row_base = t.row_base, rows_e = t.rows_e, m0 = t.m0;
 
@@ -518,6 +538,75 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
 #pragma unroll
       for (int v = 0; v < Geom<ELT>::NACC; ++v) acc[i][j][v] = 0.f;
 
+  // ---- block scales (BS only) ------------------------------------------------------------------------
+  // main: the promoted sums.  Lane l of the scale fill fetches the scale of tile row 64 * wave + l; a scale block
+  // kb of K adds as_kstep bytes to every lane's offset.  b_scale: one value per pair, a scalar load.
+  typename Geom<ELT>::Acc main_acc[BS ? MBK : 1][BS ? NBK : 1];
+  __amdgpu_buffer_rsrc_t as_rsrc = zrsrc;
+  uint32_t as_voff = 0;
+  int as_kstep = 0, bs_base = 0, bs_kstep = 0;
+  const int kblocks = nk >> 1;
+  if constexpr (BS) {
+#pragma unroll
+    for (int i = 0; i < MBK; ++i)
+#pragma unroll
+      for (int j = 0; j < NBK; ++j)
+#pragma unroll
+        for (int v = 0; v < Geom<ELT>::NACC; ++v) main_acc[i][j][v] = 0.f;
+    const KernArgs pe = kernel_args();
+    as_rsrc = make_rsrc(reinterpret_cast<const uint8_t *>(pe->a_scale), 0xffffffffll);
+    int xr = m0 + 64 * wave + lane;
+    if (xr > rows_e - 1) xr = rows_e - 1;
+    int64_t arow = row_base + xr;
+    if (pe->gather_a != nullptr) {
+      arow = pe->gather_a[row_base + xr];
+      if (pe->a_rows > 0) arow = arow < 0 ? 0 : (arow >= pe->a_rows ? pe->a_rows - 1 : arow);
+    }
+    if (pe->a_scale_layout == FLUXMI_ASCALE_BLOCK128) {  // [ceil(rows/128), K/128, 128], row in block fastest
+      as_voff = static_cast<uint32_t>(((arow >> 7) * kblocks * 128 + (arow & 127)) * 4);
+      as_kstep = 128 * 4;
+    } else {  // per expert [K/128, rows of the expert], experts back to back
+      as_voff = static_cast<uint32_t>((static_cast<int64_t>(row_base) * kblocks + xr) * 4);
+      as_kstep = rows_e * 4;
+    }
+    int n0g = t.n0;
+    split_group(n0g, pe->n, pe->ngroups);
+    const int nb = n0g >> 7, nblocks = (pe->n + 127) >> 7;
+    if (pe->b_scale_layout == FLUXMI_BSCALE_N_K) {  // [E, N/128, K/128]
+      bs_base = (e * nblocks + nb) * kblocks;
+      bs_kstep = 1;
+    } else {  // [E, K/128, N/128]
+      bs_base = e * kblocks * nblocks + nb;
+      bs_kstep = nblocks;
+    }
+  }
+  // The scale fill of scale block kb into ring slot `slot` (one instruction per wave, also past the end of K,
+  // where it reads zeros: the fill counts of the waits must hold).
+  auto scale_fill = [&](int slot, int kb) {
+    const bool in = kb < kblocks;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(in ? as_rsrc : zrsrc, (lds_ptr_t)(smem + slot * SB + SCALE_OFF + wave * 256), 4,
+                                             static_cast<int>(in ? as_voff : static_cast<uint32_t>(lane * 4)),
+                                             in ? kb * as_kstep : 0, 0, 0);
+  };
+  // End of a pair of k-steps: main += acc * (row scale * block scale of B), acc = 0.
+  auto promote = [&](int slot, int kb) {
+    if constexpr (BS) {
+      const float bsv = kernel_args()->b_scale[__builtin_amdgcn_readfirstlane(bs_base + kb * bs_kstep)];
+      const float *srow = reinterpret_cast<const float *>(smem + slot * SB + SCALE_OFF) + wm * (32 * MB) + (lane & 31);
+#pragma unroll
+      for (int i = 0; i < MBK; ++i) {
+        const float sc = srow[i * 32] * bsv;
+#pragma unroll
+        for (int j = 0; j < NBK; ++j)
+#pragma unroll
+          for (int v = 0; v < Geom<ELT>::NACC; ++v) {
+            main_acc[i][j][v] = fmaf(acc[i][j][v], sc, main_acc[i][j][v]);
+            acc[i][j][v] = 0.f;
+          }
+      }
+    }
+  };
+
   // Fragment addresses: per lane and 16-byte chunk s a base for each operand; a stage and block add a
   // compile-time offset.  LDS instructions carry 16 bits of offset, so three bases 64 KiB apart.
   const uint8_t *xfrag[3][NCH], *wfrag[3][NCH];
@@ -558,12 +647,13 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
     constexpr int e0 = u & ~1;
     // Stage u+1 has landed once the pair it belongs to is complete; fills are counted in issue order.
     if constexpr (even) {
-      FLUXMI_WAITCNT((LA - 2) * LOADS, 15);  // all but the pairs requested since the one stage u+1 is in
+      FLUXMI_WAITCNT(WAIT_EVEN, 15);  // all but the pairs requested since the one stage u+1 is in
     } else {
-      FLUXMI_WAITCNT((LA - 3) * LOADS, 15);  // ... and the half pair requested during the last step
+      FLUXMI_WAITCNT(WAIT_ODD, 15);  // ... and the half pair requested during the last step
     }
     __builtin_amdgcn_s_barrier();     // ... for every wave's share; and everybody is done reading stage u
     __builtin_amdgcn_sched_barrier(0);
+    if constexpr (BS && even) scale_fill((e0 + LA) % STG, (kbase / KBYTES + e0 + LA) >> 1);
     static_for<0, NM>([&](auto T) {
       constexpr int t = decltype(T)::value;
       static_for<0, NR>([&](auto R) {
@@ -592,6 +682,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
       mfma_slot<ELT, MBK, NBK>(t, xc, wc, acc);
       __builtin_amdgcn_sched_barrier(0);
     });
+    if constexpr (BS && !even) promote(e0 % STG, (kbase / KBYTES + e0) >> 1);
     FLUXMI_WAITCNT(63, 0);  // the fragments of the next step are in registers (requested long ago)
     __builtin_amdgcn_sched_barrier(0);
   };
@@ -599,14 +690,17 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
   // number is not a multiple of ten.
   auto step_dyn = [&](int ks, bool even, i32x4 (&xc)[MBK][NCH], i32x4 (&wc)[NBK][NCH], i32x4 (&xn)[MBK][NCH], i32x4 (&wn_)[NBK][NCH]) {
     if (even) {
-      FLUXMI_WAITCNT((LA - 2) * LOADS, 15);
+      FLUXMI_WAITCNT(WAIT_EVEN, 15);
     } else {
-      FLUXMI_WAITCNT((LA - 3) * LOADS, 15);
+      FLUXMI_WAITCNT(WAIT_ODD, 15);
     }
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
     const int e0 = even ? ks : ks - 1;
     const int rslot = (ks + 1) % STG, pslot0 = (e0 + LA) % STG, pslot1 = (e0 + LA + 1) % STG;
+    if constexpr (BS) {
+      if (even) scale_fill(pslot0, (e0 + LA) >> 1);
+    }
     static_for<0, NM>([&](auto T) {
       constexpr int t = decltype(T)::value;
       static_for<0, NR>([&](auto R) {
@@ -625,14 +719,30 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
       mfma_slot<ELT, MBK, NBK>(t, xc, wc, acc);
       __builtin_amdgcn_sched_barrier(0);
     });
+    if constexpr (BS) {
+      if (!even) promote(e0 % STG, e0 >> 1);
+    }
     FLUXMI_WAITCNT(63, 0);
     __builtin_amdgcn_sched_barrier(0);
   };
 
   // ---- prologue: k-steps 0..3 requested as two pairs, here or by the previous tile ahead of its epilogue --
   FLUXMI_WAITCNT(0, 0);  // stores of the previous tile's epilogue (and, if it requested them, the first fills)
-  if (!prefetched) issue_first_pairs<XLOADS, WLOADS>(op, smem, c);
-  FLUXMI_WAITCNT((LA - 2) * LOADS, 15);
+  if constexpr (BS) {
+    // Pair by pair like issue_first_pairs, each pair led by its scale fill.
+#pragma unroll
+    for (int s0 = 0; s0 < LA; s0 += 2) {
+      scale_fill(s0, s0 >> 1);
+#pragma unroll
+      for (int q = 0; q < LOADS; ++q) {
+        fill_any<XLOADS, WLOADS>(op, smem, c, q, s0, s0);
+        fill_any<XLOADS, WLOADS>(op, smem, c, q, s0 + 1, s0 + 1);
+      }
+    }
+  } else {
+    if (!prefetched) issue_first_pairs<XLOADS, WLOADS>(op, smem, c);
+  }
+  FLUXMI_WAITCNT(WAIT_EVEN, 15);
   __builtin_amdgcn_s_barrier();
   static_for<0, NR>([&](auto R) { read_one(std::integral_constant<int, 0>{}, R, xa, wa); });
   FLUXMI_WAITCNT(63, 0);  // in registers before the first step's barrier lets anyone refill that slot
@@ -679,24 +789,29 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
     int n0 = t.n0;
     const int g = split_group(n0, pe->n, pe->ngroups);
     const int wcol0 = n0 + wn * (32 * NB);
-    const bool full = wrow0 + 32 * MB <= rows_e && wcol0 + 32 * NB <= pe->n && pe->scatter_d == nullptr;
+    const bool full = wrow0 + 32 * MB <= rows_e && wcol0 + 32 * NB <= pe->n && pe->scatter_d == nullptr &&
+                      pe->accumulate == 0;
     const bool out_f32 = pe->d_fp32 != 0;
     const bool scaled = !(c.scalar == 1.f && pe->alpha[g] == nullptr && pe->row_scale == nullptr && pe->col_scale == nullptr);
-    if (full && !scaled) {
-      if (out_f32) store_tile<ELT, MB, NB, true, true, false>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, acc);
-      else store_tile<ELT, MB, NB, true, false, false>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, acc);
-    } else if (full) {
-      if (out_f32) store_tile<ELT, MB, NB, true, true, true>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, acc);
-      else store_tile<ELT, MB, NB, true, false, true>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, acc);
-    } else {
-      if (out_f32) store_tile<ELT, MB, NB, false, true, true>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, acc);
-      else store_tile<ELT, MB, NB, false, false, true>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, acc);
-    }
+    auto store = [&](const typename Geom<ELT>::Acc (&res)[MBK][NBK]) {
+      if (full && !scaled) {
+        if (out_f32) store_tile<ELT, MB, NB, true, true, false>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, res);
+        else store_tile<ELT, MB, NB, true, false, false>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, res);
+      } else if (full) {
+        if (out_f32) store_tile<ELT, MB, NB, true, true, true>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, res);
+        else store_tile<ELT, MB, NB, true, false, true>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, res);
+      } else {
+        if (out_f32) store_tile<ELT, MB, NB, false, true, true>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, res);
+        else store_tile<ELT, MB, NB, false, false, true>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, res);
+      }
+    };
+    if constexpr (BS) store(main_acc);
+    else store(acc);
   }
   __builtin_amdgcn_s_barrier();  // the LDS windows are free again before the next tile's fills start
 }
 
-template <int ELT>
+template <int ELT, bool BS = false>
 __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmParams p) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];  // STAGES x (X tile | W tile)
 
@@ -770,11 +885,12 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
   // Full rounds run whole macro tiles.  The tiles of the last, partly filled round are cut into
   // `pieces` parts (2 pieces of 256x128, or 4 of 128x128) when that still fits one round, so that the
   // chip does not idle while a fraction of the CUs finishes whole tiles.
-  const int full_items = (total_tiles / grid) * grid;
+  // Block-scaled launches run every tile as two 256 x 128 pieces (one column block of B's scales each).
+  const int full_items = BS ? 0 : (total_tiles / grid) * grid;
   const int rem_tiles = total_tiles - full_items;
   const bool cut_tail = (p.sched_flags & FLUXMI_SCHED_WHOLE_TAIL_TILES) == 0;
   const bool half_tiles = (p.sched_flags & FLUXMI_SCHED_NO_HALF_TILES) == 0;
-  const int pieces = !cut_tail ? 1 : (rem_tiles * 4 <= grid ? 4 : (rem_tiles * 2 <= grid ? 2 : 1));
+  const int pieces = BS ? 2 : (!cut_tail ? 1 : (rem_tiles * 4 <= grid ? 4 : (rem_tiles * 2 <= grid ? 2 : 1)));
   const int total_items = full_items + rem_tiles * pieces;
 
   // ---- schedule: walk the experts once, in step with this workgroup's increasing tile ids ----------
@@ -850,20 +966,24 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
   while (cur.kind != -2) {
     item += grid;
     const TileDesc next = locate(item);
-    if (cur.kind == 0) gemm_tile<ELT, 4, 4>(p, smem, c, cur, next, pf);
-    else if (cur.kind == 1) gemm_tile<ELT, 2, 4>(p, smem, c, cur, next, pf);
-    else if (cur.kind == 2) gemm_tile<ELT, 4, 2>(p, smem, c, cur, next, pf);
-    else if (cur.kind == 3) gemm_tile<ELT, 2, 2>(p, smem, c, cur, next, pf);
+    if constexpr (BS) {
+      if (cur.kind == 2) gemm_tile<ELT, 4, 2, true>(p, smem, c, cur, next, pf);
+    } else {
+      if (cur.kind == 0) gemm_tile<ELT, 4, 4>(p, smem, c, cur, next, pf);
+      else if (cur.kind == 1) gemm_tile<ELT, 2, 4>(p, smem, c, cur, next, pf);
+      else if (cur.kind == 2) gemm_tile<ELT, 4, 2>(p, smem, c, cur, next, pf);
+      else if (cur.kind == 3) gemm_tile<ELT, 2, 2>(p, smem, c, cur, next, pf);
+    }
     cur = next;
   }
 }
 
-template <int ELT>
+template <int ELT, bool BS = false>
 int launch_mfma(const GemmParams &p, int grid, hipStream_t s) {
   static std::atomic<uint64_t> lds_done{0};
-  const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(grouped_gemm_mfma_kernel<ELT>), LDS_BYTES, lds_done);
+  const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(grouped_gemm_mfma_kernel<ELT, BS>), LDS_BYTES, lds_done);
   if (rc != FLUXMI_OK) return rc;
-  hipLaunchKernelGGL((grouped_gemm_mfma_kernel<ELT>), dim3(grid), dim3(NTHREADS), LDS_BYTES, s, p);
+  hipLaunchKernelGGL((grouped_gemm_mfma_kernel<ELT, BS>), dim3(grid), dim3(NTHREADS), LDS_BYTES, s, p);
   return FLUXMI_OK;
 }
 

@@ -113,6 +113,92 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor> moe_route
   return {splits, scatter, gather, topk_index};
 }
 
+// ------------------------------------------------------------------------------------------------
+// Block-scaled fp8 GEMM
+// ------------------------------------------------------------------------------------------------
+BlockScaleGemm::BlockScaleGemm(at::ScalarType input_dtype, at::ScalarType weight_dtype, at::ScalarType output_dtype,
+                               int32_t /*num_streams*/)
+    : input_dtype_(input_dtype), weight_dtype_(weight_dtype), output_dtype_(output_dtype) {
+  TORCH_CHECK(is_fp8(input_dtype) && is_fp8(weight_dtype), "BlockScaleGemm: input and weight must be float8_e4m3fn");
+  TORCH_CHECK(output_dtype == at::kBFloat16 || output_dtype == at::kFloat,
+              "BlockScaleGemm: output dtype must be bfloat16 or float32, got ", output_dtype);
+}
+
+static torch::Tensor blockscale_run(const torch::Tensor &input, const torch::Tensor &weight3, const torch::Tensor &splits_cpu,
+                                    std::optional<torch::Tensor> output, const torch::Tensor &input_scale,
+                                    int32_t a_layout, const torch::Tensor &weight_scale, int32_t b_layout,
+                                    at::ScalarType out_dtype) {
+  const int64_t m = input.size(0), k = input.size(1), e = weight3.size(0), n = weight3.size(1);
+  TORCH_CHECK(weight3.size(2) == k, "weight 2-dim mismatch: ", weight3.size(2), " != ", k);
+  TORCH_CHECK(k % kBlock == 0, "K must be a multiple of 128, got ", k);
+  FLUX_AMD_CHECK_INPUT(input_scale, at::kFloat);
+  FLUX_AMD_CHECK_INPUT(weight_scale, at::kFloat);
+  const int64_t kb = k / kBlock, nb = (n + kBlock - 1) / kBlock;
+  TORCH_CHECK(weight_scale.numel() == e * nb * kb, "weight_scale has ", weight_scale.numel(), " entries, expected ",
+              e * nb * kb);
+  const int64_t want_a = a_layout == FLUXMI_ASCALE_BLOCK128 ? (m + kBlock - 1) / kBlock * kBlock * kb : m * kb;
+  TORCH_CHECK(input_scale.numel() == want_a, "input_scale has ", input_scale.numel(), " entries, expected ", want_a);
+  torch::Tensor out;
+  if (output.has_value()) {
+    out = *output;
+    FLUX_AMD_CHECK_INPUT(out, out_dtype);
+    FLUX_AMD_CHECK_2D(out, m, n);
+  } else {
+    out = torch::empty({m, n}, input.options().dtype(out_dtype));
+  }
+  if (m == 0) return out;
+  torch::Tensor splits_dev = splits_cpu.to(at::kInt).to(input.device(), /*non_blocking=*/true);
+  fluxmi_grouped_gemm_args args{};
+  args.dtype = FLUXMI_FP8_E4M3;
+  args.nexperts = static_cast<int32_t>(e);
+  args.max_rows = static_cast<int32_t>(m);
+  args.n = static_cast<int32_t>(n);
+  args.k = static_cast<int32_t>(k);
+  args.a_rows = static_cast<int32_t>(m);
+  args.a = input.data_ptr();
+  args.b = weight3.data_ptr();
+  args.d = out.data_ptr();
+  args.splits = splits_dev.data_ptr<int32_t>();
+  args.scalar_scale = 1.0f;
+  args.d_fp32 = out_dtype == at::kFloat ? 1 : 0;
+  check_status(fluxmi_grouped_gemm_blockscale(&args, input_scale.data_ptr<float>(), a_layout,
+                                              weight_scale.data_ptr<float>(), b_layout, current_stream()),
+               "fluxmi_grouped_gemm_blockscale");
+  return out;
+}
+
+torch::Tensor BlockScaleGemm::forward(torch::Tensor input, torch::Tensor weight, std::optional<torch::Tensor> bias,
+                                      std::optional<torch::Tensor> output, std::optional<torch::Tensor> input_scale,
+                                      std::optional<torch::Tensor> weight_scale) {
+  TORCH_CHECK(!bias.has_value(), "BlockScaleGemm: bias is not supported");  // as in the reference
+  TORCH_CHECK(input_scale.has_value() && weight_scale.has_value(), "BlockScaleGemm: input_scale and weight_scale are required");
+  FLUX_AMD_CHECK_INPUT(input, input_dtype_);
+  FLUX_AMD_CHECK_INPUT(weight, weight_dtype_);
+  FLUX_AMD_CHECK_NDIM(input, 2);
+  FLUX_AMD_CHECK_NDIM(weight, 2);
+  torch::Tensor splits = torch::full({1}, input.size(0), at::TensorOptions().dtype(at::kInt));
+  return blockscale_run(input, weight.unsqueeze(0), splits, output, *input_scale, FLUXMI_ASCALE_BLOCK128, *weight_scale,
+                        FLUXMI_BSCALE_N_K, output_dtype_);
+}
+
+torch::Tensor BlockScaleGemm::forward_grouped(torch::Tensor input, torch::Tensor input_splits, torch::Tensor weight,
+                                              std::optional<torch::Tensor> bias, std::optional<torch::Tensor> output,
+                                              torch::Tensor input_scale, torch::Tensor weight_scale) {
+  TORCH_CHECK(!bias.has_value(), "BlockScaleGemm: bias is not supported");
+  FLUX_AMD_CHECK_INPUT(input, input_dtype_);
+  FLUX_AMD_CHECK_INPUT(weight, weight_dtype_);
+  FLUX_AMD_CHECK_NDIM(input, 2);
+  FLUX_AMD_CHECK_NDIM(weight, 3);
+  FLUX_AMD_CHECK_NDIM(input_splits, 1);
+  TORCH_CHECK(!input_splits.is_cuda(), "input splits is not on cpu");
+  TORCH_CHECK(input_splits.size(0) == weight.size(0), "splits 0-dim mismatch: ", input_splits.size(0), " != ",
+              weight.size(0));
+  TORCH_CHECK(input_splits.sum().item<int64_t>() <= input.size(0), "input_splits sum exceeds the rows of input");
+  const int32_t a_layout = input_scale.dim() == 3 ? FLUXMI_ASCALE_BLOCK128 : FLUXMI_ASCALE_EXPERT_K_M;
+  const int32_t b_layout = weight_scale.dim() == 3 ? FLUXMI_BSCALE_N_K : FLUXMI_BSCALE_K_N;
+  return blockscale_run(input, weight, input_splits, output, input_scale, a_layout, weight_scale, b_layout, output_dtype_);
+}
+
 torch::Tensor calc_scatter_index(torch::Tensor choosed_experts, torch::Tensor splits) {
   FLUX_AMD_CHECK_INPUT(choosed_experts, at::kInt);
   FLUX_AMD_CHECK_INPUT(splits, at::kInt);

@@ -287,6 +287,12 @@ GemmGroupedV3GatherRS::GemmGroupedV3GatherRS(int64_t total_num_experts, int64_t 
   TORCH_CHECK(max_input_groups >= 1 && max_input_groups <= 4, "max_input_groups must be in [1, 4]");
   const char *env = std::getenv("FLUX_AMD_INTER_DTYPE");
   inter_fp32_ = !(env != nullptr && std::string(env) == "bf16");
+  // Where the top-k reduction happens: in the GEMM's epilogue (atomic adds into an fp32 [T, N] buffer, the
+  // reference's fused form) or in a gather-reduce kernel after the GEMM (deterministic for every top-k).
+  const char *red = std::getenv("FLUX_AMD_LAYER1_REDUCE");
+  if (red != nullptr && std::string(red) == "fused") fused_mode_ = 1;
+  else if (red != nullptr && std::string(red) == "twopass") fused_mode_ = 2;
+  else TORCH_CHECK(red == nullptr || std::string(red).empty(), "FLUX_AMD_LAYER1_REDUCE must be 'fused' or 'twopass', got ", red);
 }
 
 void GemmGroupedV3GatherRS::lazy_init(const torch::Tensor &like) {
@@ -298,6 +304,7 @@ void GemmGroupedV3GatherRS::lazy_init(const torch::Tensor &like) {
   auto opts = like.options().dtype(inter_fp32_ ? at::kFloat : at::kBFloat16);
   for (int64_t g = 0; g < max_input_groups_; ++g) inter_.push_back(torch::zeros({max_m_, n_dim_}, opts));
   splits_dev_ = torch::empty({num_experts_}, like.options().dtype(at::kInt));
+  token_of_row_ = torch::empty({max_m_}, like.options().dtype(at::kInt));
 }
 
 torch::Tensor GemmGroupedV3GatherRS::forward_impl(
@@ -345,6 +352,9 @@ torch::Tensor GemmGroupedV3GatherRS::forward_impl(
   if (global_m == 0) return out;
   splits_dev_.copy_(splits_cpu.contiguous(), /*non_blocking=*/true);
 
+  // One input group, an fp32 scratch at hand and the fused form asked for: the reduction runs in the GEMM's
+  // epilogue.  (By shape nothing selects it yet: the two-pass form is the default everywhere.)
+  const bool fused = fused_mode_ == 1 && groups == 1 && inter_fp32_;
   std::vector<const void *> group_ptrs;
   for (size_t g = 0; g < groups; ++g) {
     const float *alpha = nullptr, *row = nullptr, *col = nullptr, *scalar = nullptr;
@@ -366,6 +376,35 @@ torch::Tensor GemmGroupedV3GatherRS::forward_impl(
       else TORCH_CHECK(false, "input_scale must be [1] or [M]");
     }
     if (row_holder.defined()) row = row_holder.data_ptr<float>();
+    if (fused) {
+      token_of_row_.fill_(-1);  // sorted rows that no routing entry names are skipped by the epilogue
+      check_status(fluxmi_moe_gather_index(routing_idx.data_ptr<int32_t>(), static_cast<int32_t>(global_m),
+                                           static_cast<int32_t>(topk_), token_of_row_.data_ptr<int32_t>(), nullptr,
+                                           current_stream()),
+                   "fluxmi_moe_gather_index");
+      fluxmi_grouped_gemm_args args{};
+      args.dtype = to_fluxmi_dtype(inputs[g].scalar_type());
+      args.nexperts = static_cast<int32_t>(num_experts_);
+      args.max_rows = static_cast<int32_t>(m);
+      args.n = static_cast<int32_t>(n_dim_);
+      args.k = static_cast<int32_t>(k);
+      args.a_rows = static_cast<int32_t>(m);
+      args.a = inputs[g].data_ptr();
+      args.b = weights[g].data_ptr();
+      args.splits = splits_dev_.data_ptr<int32_t>();
+      args.alpha = alpha;
+      args.row_scale = row;
+      args.col_scale = col;
+      args.scalar_scale = 1.0f;
+      args.scalar_scale_dev = scalar;
+      apply_launch_tuning(args, 1, sm_margin);
+      check_status(fluxmi_grouped_gemm_topk_reduce(&args, token_of_row_.data_ptr<int32_t>(), static_cast<int32_t>(ntokens),
+                                                   out.data_ptr(), inter_[0].data_ptr(),
+                                                   static_cast<size_t>(inter_[0].numel()) * 4, current_stream()),
+                   "fluxmi_grouped_gemm_topk_reduce");
+      if (with_stream_sync) c10::hip::getCurrentHIPStream().synchronize();
+      return out;
+    }
     run_grouped_gemm(inputs[g], weights[g], splits_dev_, inter_[g], nullptr, m, alpha, row, col, scalar, sm_margin);
     group_ptrs.push_back(inter_[g].data_ptr());
   }

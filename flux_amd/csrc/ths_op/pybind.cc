@@ -111,6 +111,22 @@ PYBIND11_MODULE(flux_ths_pybind, m) {
       .def(py::init<torch::Tensor, int64_t>(), py::arg("weight"), py::arg("num_experts"))
       .def("forward", &GemmGroupedV3::forward, py::arg("input"), py::arg("splits_cpu"));
 
+  // src/pybind/gemm_only.cc:77-139 (forward and forward_grouped; the weight-gradient and multi-stream methods are
+  // not built)
+  py::class_<BlockScaleGemm>(m, "BlockScaleGemm")
+      .def(py::init([](py::object input_dtype, py::object weight_dtype, py::object output_dtype, int32_t num_streams) {
+             const at::ScalarType in = to_dtype(input_dtype);
+             return new BlockScaleGemm(in, to_dtype(weight_dtype), output_dtype.is_none() ? in : to_dtype(output_dtype),
+                                       num_streams);
+           }),
+           py::arg("input_dtype"), py::arg("weight_dtype"), py::arg("output_dtype") = py::none(),
+           py::arg("num_streams") = 2)
+      .def("forward", &BlockScaleGemm::forward, py::arg("input"), py::arg("weight"), py::arg("bias") = py::none(),
+           py::arg("output") = py::none(), py::arg("input_scale") = py::none(), py::arg("weight_scale") = py::none())
+      .def("forward_grouped", &BlockScaleGemm::forward_grouped, py::arg("input"), py::arg("input_splits"),
+           py::arg("weight"), py::arg("bias") = py::none(), py::arg("output") = py::none(),
+           py::arg("input_scale") = py::none(), py::arg("weight_scale") = py::none());
+
   py::class_<Quantization>(m, "Quantization")
       .def(py::init([](py::object input_dtype, py::object output_dtype, int32_t num_streams) {
              return new Quantization(to_dtype(input_dtype), to_dtype(output_dtype), num_streams);

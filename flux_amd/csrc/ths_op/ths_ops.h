@@ -73,8 +73,10 @@ class GemmGroupedV3GatherRS {
   void lazy_init(const torch::Tensor &like);
   int64_t num_experts_, max_m_, n_dim_, topk_, max_input_groups_;
   bool inter_fp32_ = true;
+  int fused_mode_ = 0;  // 0: by shape, 1: always the fused epilogue reduce, 2: always GEMM + gather-reduce
   std::vector<torch::Tensor> inter_;
   torch::Tensor splits_dev_;
+  torch::Tensor token_of_row_;  // inverse of routing_idx (the token of each sorted row), for the fused reduce
 };
 
 class GemmGroupedV3 {
@@ -84,6 +86,30 @@ class GemmGroupedV3 {
 
  private:
   torch::Tensor weight_;
+};
+
+// Block-scaled fp8 GEMM of the reference (src/comm_none/ths_op/blockscale_gemm.h:24-94): the forward
+// products, dense and grouped.  wgrad / the multi-stream variants (training-time weight gradients, per-expert
+// streams) are not on this path and are not built.
+class BlockScaleGemm {
+ public:
+  BlockScaleGemm(at::ScalarType input_dtype, at::ScalarType weight_dtype, at::ScalarType output_dtype,
+                 int32_t num_streams);
+  // input [M, K] e4m3, weight [N, K] e4m3, input_scale [ceil(M/128), K/128, 128] (what
+  // Quantization::quantize_vector_blockwise returns), weight_scale [ceil(N/128), K/128].
+  torch::Tensor forward(torch::Tensor input, torch::Tensor weight, std::optional<torch::Tensor> bias,
+                        std::optional<torch::Tensor> output, std::optional<torch::Tensor> input_scale,
+                        std::optional<torch::Tensor> weight_scale);
+  // input [M, K] sorted by expert, input_splits host [E], weight [E, N, K].  Scales either in the reference's
+  // operand layouts (1-D tensors: per expert [K/128, M_e] back to back; per expert [K/128, N/128]:
+  // blockscale_gemm.cc:703-722) or as the quantisation ops return them (3-D tensors: input_scale
+  // [ceil(M/128), K/128, 128] over the sorted rows, weight_scale [E, N/128, K/128]).
+  torch::Tensor forward_grouped(torch::Tensor input, torch::Tensor input_splits, torch::Tensor weight,
+                                std::optional<torch::Tensor> bias, std::optional<torch::Tensor> output,
+                                torch::Tensor input_scale, torch::Tensor weight_scale);
+
+ private:
+  at::ScalarType input_dtype_, weight_dtype_, output_dtype_;
 };
 
 class Quantization {

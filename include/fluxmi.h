@@ -148,6 +148,58 @@ int fluxmi_grouped_gemm(const fluxmi_grouped_gemm_args *args, void *workspace,
  * shapes only); callers use this to assert they are not on the generic kernel. */
 int fluxmi_grouped_gemm_kernel_kind(const fluxmi_grouped_gemm_args *args);
 
+/* ------------------------------------------------------------------------------------------------
+ * Top-k reduction fused into the grouped GEMM's epilogue (layer1 in one pass, no [M, N] intermediate):
+ *
+ *   out[t, n] = bf16( sum over sorted rows r with token_of_row[r] == t of
+ *                       acc[r, n] * alpha[e] * row_scale[r] * col_scale[e, n] * scalar_scale )
+ *
+ * Stands in for the fused GEMM + top-k reduce kernel of `GemmGroupedV3GatherRS`
+ * (src/moe_gather_rs/sm90_gemm_array_threadblock_specialized.hpp:1306-1409 reduce, :1916-2086 GEMM).  The
+ * epilogue adds each scaled fp32 result into row token_of_row[r] of a fp32 [ntokens, N] workspace with
+ * hardware float atomics; a pass before clears the workspace, a pass after rounds it to bf16 `out`.
+ * `token_of_row` is the device array gather_index ([max_rows] int32: the token of each sorted row; entries
+ * outside [0, ntokens) are skipped).  args->d, d_fp32 and scatter_d are not used (scatter_d must be NULL);
+ * every other member means what it means for fluxmi_grouped_gemm.  With top-2 the result does not depend on the
+ * order of the additions; with more terms per token the last bits can differ from run to run (fp32 addition is
+ * not associative), far inside the 1e-2 bound.  The two-pass form (fluxmi_grouped_gemm with d_fp32 = 1, then
+ * fluxmi_topk_gather_reduce) is deterministic for every top-k.
+ * ---------------------------------------------------------------------------------------------- */
+size_t fluxmi_grouped_gemm_topk_reduce_workspace_bytes(int32_t ntokens, int32_t n);
+int fluxmi_grouped_gemm_topk_reduce(const fluxmi_grouped_gemm_args *args, const int32_t *token_of_row,
+                                    int32_t ntokens, void *out, void *workspace, size_t workspace_bytes,
+                                    void *stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Block-scaled fp8 grouped GEMM (DeepSeek-style 1 x 128 activation scales, 128 x 128 weight scales):
+ *
+ *   acc[r, n] = sum over scale blocks kb of K ( a_scale[row, kb] * b_scale[e, n / 128, kb] *
+ *                 sum_{k in block kb} float(A[row, k]) * float(B[e, n, k]) ),   row = gather_a ? gather_a[r] : r
+ *   D as for fluxmi_grouped_gemm (alpha, row_scale, col_scale, scalar scales, scatter_d, d_fp32 all apply).
+ *
+ * Stands in for the kernels behind `BlockScaleGemm::forward_grouped` / `forward`
+ * (src/comm_none/ths_op/blockscale_gemm.cc:648-782, arguments include/flux/args/comm_none.h:169-184; reference
+ * semantics test/python/gemm_only/test_blockwise_scale_gemm_only.py:200-262): the products of each 128 of K are
+ * summed exactly in fp32 and promoted into the result with their scales.  dtype must be FLUXMI_FP8_E4M3 and
+ * K % 128 == 0.  Scale layouts (both are the `scale_inv` outputs of the quantisation entry points below or the
+ * reference's own operand layouts):
+ *   a_scale  FLUXMI_ASCALE_BLOCK128: [ceil(rows_a / 128), K / 128, 128], the row inside its block of 128 rows
+ *            fastest — what fluxmi_quant_e4m3_block128 / quantize_vector_blockwise write for the A matrix
+ *            (indexed by the row of A that is read, so it works with gather_a);
+ *            FLUXMI_ASCALE_EXPERT_K_M: experts back to back, each [K / 128, rows of the expert] (rows fastest),
+ *            expert e starting at float offset offsets[e] * K / 128 — what forward_grouped takes
+ *            (blockscale_gemm.cc:717-718); not with gather_a.
+ *   b_scale  FLUXMI_BSCALE_N_K: [E, ceil(N / 128), K / 128] — what fluxmi_quant_e4m3_square writes for B;
+ *            FLUXMI_BSCALE_K_N: [E, K / 128, ceil(N / 128)] — what forward_grouped takes (:719-721).
+ * ---------------------------------------------------------------------------------------------- */
+#define FLUXMI_ASCALE_BLOCK128 0
+#define FLUXMI_ASCALE_EXPERT_K_M 1
+#define FLUXMI_BSCALE_N_K 0
+#define FLUXMI_BSCALE_K_N 1
+int fluxmi_grouped_gemm_blockscale(const fluxmi_grouped_gemm_args *args, const float *a_scale,
+                                   int32_t a_scale_layout, const float *b_scale, int32_t b_scale_layout,
+                                   void *stream);
+
 /* The same rows times `ngroups` (1..4) weight tensors in ONE launch, each group with an output of its own:
  * `GemmGroupedV3AGScatterOp::forward_multiple_weights` (gate and up projections sharing the gathered
  * A tiles; src/moe_ag_scatter/ths_op/gemm_grouped_v3_ag_scatter.cc:375-395).  b, d and alpha are

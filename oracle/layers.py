@@ -120,3 +120,39 @@ def fp8_grouped_gemm_fp32(q_a, a_scale_inv, q_w, w_scale_inv, split, row_weight=
     a = q_a.to(torch.float32) * a_scale_inv.to(torch.float32)[:, None]
     w = q_w.to(torch.float32) * w_scale_inv.to(torch.float32)[:, :, None]
     return grouped_gemm_fp32(a, w, split, row_scale=row_weight)
+
+
+def fp8_blockscale_grouped_gemm_fp32(q_a, a_scale, q_w, w_scale, split, block=128):
+    """Block-scaled fp8 grouped GEMM, dequantise-by-block form: A[r, k] = float(q_a[r, k]) * a_scale[r, k // 128],
+    W[e, n, k] = float(q_w[e, n, k]) * w_scale[e, n // 128, k // 128], then the fp32 grouped matmul.  Equal, up to
+    fp32 summation order, to the promotion form of the reference's kernels and test
+    (test/python/gemm_only/test_blockwise_scale_gemm_only.py:200-262: acc_per_tile = input_scale * weight_scale *
+    matmul over one K block, summed over the K blocks; include/flux/args/comm_none.h:169-184).
+    a_scale: [rows, K/128] (plain row-major), w_scale: [E, ceil(N/128), K/128]."""
+    rows, k = q_a.shape
+    e_cnt, n, _ = q_w.shape
+    kb = k // block
+    a = q_a.to(torch.float32).reshape(rows, kb, block) * a_scale.to(torch.float32)[:, :, None]
+    w_rows = torch.repeat_interleave(w_scale.to(torch.float32), block, dim=1)[:, :n, :]      # [E, N, K/128]
+    w = q_w.to(torch.float32).reshape(e_cnt, n, kb, block) * w_rows[:, :, :, None]
+    return grouped_gemm_fp32(a.reshape(rows, k), w.reshape(e_cnt, n, k), split)
+
+
+def a_scale_to_block128(a_scale):
+    """[rows, K/128] -> the permuted layout [ceil(rows/128), K/128, 128] (row inside its block fastest) that the
+    reference's quantize_vector_blockwise writes (src/quantization/ths_op/quantization.cc:75-145); rows past the end
+    hold zeros."""
+    rows, kb = a_scale.shape
+    nb = (rows + 127) // 128
+    out = torch.zeros(nb * 128, kb, dtype=a_scale.dtype)
+    out[:rows] = a_scale
+    return out.reshape(nb, 128, kb).permute(0, 2, 1).contiguous()
+
+
+def a_scale_to_expert_k_m(a_scale, split):
+    """[rows, K/128] -> experts back to back, each [K/128, rows of the expert] (rows fastest): the operand layout of
+    BlockScaleGemm::forward_grouped (src/comm_none/ths_op/blockscale_gemm.cc:717-718; built the same way in
+    test/python/gemm_only/test_blockwise_scale_gemm_only.py:748-753)."""
+    off = routing.offsets(np.asarray(split))
+    parts = [a_scale[int(off[e]):int(off[e + 1])].t().contiguous().reshape(-1) for e in range(len(split))]
+    return torch.cat(parts) if parts else a_scale.reshape(-1)

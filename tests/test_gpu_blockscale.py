@@ -1,0 +1,168 @@
+"""GPU parity, block-scaled fp8 grouped GEMM (1 x 128 activation scales, 128 x 128 weight scales, promotion every
+128 of K) against the dequantise-by-block oracle: products of e4m3 values and their block sums are exact in fp32, so
+only the order of the fp32 additions differs (tight bound); at the C5 shapes, with operands quantised on the GPU,
+the bound is the benchmark's 3e-2 relative Frobenius error."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import configs, layers, routing
+
+pytestmark = pytest.mark.gpu
+
+
+def random_splits(rng, experts, rows, empty=()):
+    p = rng.random(experts) + 0.05
+    for e in empty:
+        p[e] = 0
+    return rng.multinomial(rows, p / p.sum()).astype(np.int32)
+
+
+def make_case(seed, experts, rows, n, k, empty=()):
+    rng = np.random.default_rng(seed)
+    g = torch.Generator().manual_seed(seed)
+    split = random_splits(rng, experts, rows, empty)
+    qa = torch.randn(rows, k, generator=g).to(torch.float8_e4m3fn)
+    qw = torch.randn(experts, n, k, generator=g).to(torch.float8_e4m3fn)
+    sa = torch.rand(rows, k // 128, generator=g) + 0.5
+    sw = torch.rand(experts, (n + 127) // 128, k // 128, generator=g) + 0.5
+    return split, qa, qw, sa, sw
+
+
+@pytest.mark.parametrize("experts,rows,n,k,seed,empty", [
+    (1, 256, 128, 128, 0, ()), (1, 300, 264, 256, 1, ()), (4, 1000, 512, 384, 2, ()), (8, 2048, 1024, 1024, 3, (0, 5)),
+    (3, 700, 1408, 2048, 4, (1,)), (16, 900, 256, 640, 5, (2, 3, 15)), (2, 17, 8, 128, 6, ()), (5, 1, 520, 1280, 7, (0, 1, 2, 4)),
+    (2, 600, 640, 1792, 8, ()), (3, 5000, 4096, 512, 9, ()), (1, 130, 136, 2816, 10, ())])
+def test_blockscale_against_oracle_both_layouts(experts, rows, n, k, seed, empty):
+    from flux_amd import capi
+    print(f"[case] blockscale E={experts} rows={rows} N={n} K={k} empty={empty}", flush=True)
+    split, qa, qw, sa, sw = make_case(seed, experts, rows, n, k, empty)
+    ref = layers.fp8_blockscale_grouped_gemm_fp32(qa, sa, qw, sw, split)
+    sp = torch.from_numpy(split).cuda()
+    tol = dict(rtol=1e-4, atol=2e-3 * k ** 0.5)
+    # the quantisation ops' layouts: a_scale [rows/128, K/128, 128], b_scale [E, N/128, K/128]
+    out = capi.grouped_gemm_blockscale(qa.cuda(), qw.cuda(), sp, layers.a_scale_to_block128(sa).cuda(), sw.cuda(),
+                                       out_dtype=torch.float32).cpu()
+    assert torch.allclose(out, ref, **tol), float((out - ref).abs().max())
+    # the reference op's operand layouts: a_scale per expert [K/128, M_e], b_scale [E, K/128, N/128]
+    out2 = capi.grouped_gemm_blockscale(qa.cuda(), qw.cuda(), sp, layers.a_scale_to_expert_k_m(sa, split).cuda(),
+                                        sw.transpose(1, 2).contiguous().cuda(), capi.ASCALE_EXPERT_K_M, capi.BSCALE_K_N,
+                                        out_dtype=torch.float32).cpu()
+    assert torch.equal(out2, out)
+    # bf16 output: one more rounding
+    outb = capi.grouped_gemm_blockscale(qa.cuda(), qw.cuda(), sp, layers.a_scale_to_block128(sa).cuda(), sw.cuda())
+    assert outb.dtype == torch.bfloat16
+    assert torch.allclose(outb.float().cpu(), ref, rtol=1e-2, atol=1e-2 * float(ref.abs().max()))
+
+
+def test_blockscale_with_gather_scatter_and_epilogue_scales():
+    from flux_amd import capi
+    rng = np.random.default_rng(21)
+    g = torch.Generator().manual_seed(21)
+    tokens, topk, experts, k, n = 300, 3, 6, 512, 392
+    choosed = np.stack([rng.permutation(experts)[:topk] for _ in range(tokens)]).astype(np.int32)
+    split = routing.splits(choosed, experts)
+    gi, _ = routing.gather_index(routing.scatter_index_stable(choosed, experts), topk)
+    m = tokens * topk
+    qx = torch.randn(tokens, k, generator=g).to(torch.float8_e4m3fn)
+    qw = torch.randn(experts, n, k, generator=g).to(torch.float8_e4m3fn)
+    sx = torch.rand(tokens, k // 128, generator=g) + 0.5          # scales belong to the rows of A (tokens)
+    sw = torch.rand(experts, (n + 127) // 128, k // 128, generator=g) + 0.5
+    tw = torch.rand(m, generator=g) + 0.5
+    alpha = torch.rand(experts, generator=g) + 0.5
+    gl = torch.as_tensor(gi, dtype=torch.long)
+    ref = layers.fp8_blockscale_grouped_gemm_fp32(qx[gl], sx[gl], qw, sw, split)
+    eor = torch.as_tensor(routing.expert_of_row(split), dtype=torch.long)
+    ref = ref * tw[:, None] * alpha[eor][:, None]
+    perm = torch.randperm(m, generator=g).to(torch.int32)
+    ref_s = torch.zeros_like(ref)
+    ref_s[perm.long()] = ref
+    out = capi.grouped_gemm_blockscale(qx.cuda(), qw.cuda(), torch.from_numpy(split).cuda(),
+                                       layers.a_scale_to_block128(sx).cuda(), sw.cuda(), gather_a=torch.from_numpy(gi).cuda(),
+                                       scatter_d=perm.cuda(), row_scale=tw.cuda(), alpha=alpha.cuda(),
+                                       out_dtype=torch.float32).cpu()
+    assert torch.allclose(out, ref_s, rtol=1e-4, atol=2e-3 * k ** 0.5), float((out - ref_s).abs().max())
+
+
+def test_blockscale_generic_kernel_and_argument_errors():
+    from flux_amd import capi
+    split, qa, qw, sa, sw = make_case(31, 2, 40, 50, 256)       # N % 4 != 0: the generic kernel
+    ref = layers.fp8_blockscale_grouped_gemm_fp32(qa, sa, qw, sw, split)
+    sp = torch.from_numpy(split).cuda()
+    out = capi.grouped_gemm_blockscale(qa.cuda(), qw.cuda(), sp, layers.a_scale_to_block128(sa).cuda(), sw.cuda(),
+                                       out_dtype=torch.float32).cpu()
+    assert torch.allclose(out, ref, rtol=1e-4, atol=1e-2)
+    out2 = capi.grouped_gemm_blockscale(qa.cuda(), qw.cuda(), sp, layers.a_scale_to_expert_k_m(sa, split).cuda(),
+                                        sw.transpose(1, 2).contiguous().cuda(), capi.ASCALE_EXPERT_K_M, capi.BSCALE_K_N,
+                                        out_dtype=torch.float32).cpu()
+    assert torch.allclose(out2, ref, rtol=1e-4, atol=1e-2)
+    with pytest.raises(RuntimeError, match="multiple of 128"):
+        capi.grouped_gemm_blockscale(qa[:, :192].contiguous().cuda(), qw[:, :, :192].contiguous().cuda(), sp,
+                                     sa.cuda(), sw.cuda())
+    bf = torch.zeros(40, 256, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(RuntimeError, match="fp8"):
+        capi.grouped_gemm_blockscale(bf, torch.zeros(2, 52, 256, dtype=torch.bfloat16, device="cuda"), sp, sa.cuda(), sw.cuda())
+    with pytest.raises(RuntimeError, match="gather_a"):
+        capi.grouped_gemm_blockscale(qa.cuda(), qw.cuda(), sp, sa.cuda(), sw.cuda(), capi.ASCALE_EXPERT_K_M, capi.BSCALE_N_K,
+                                     gather_a=torch.zeros(40, dtype=torch.int32, device="cuda"))
+
+
+def sampled_rows(split, per_expert, rng):
+    off = routing.offsets(split)
+    rows = []
+    for e in range(len(split)):
+        lo, hi = int(off[e]), int(off[e + 1])
+        if hi > lo:
+            pick = {lo, hi - 1, lo + (hi - lo) // 2}
+            pick.update(int(v) for v in rng.integers(lo, hi, size=per_expert))
+            rows.extend(sorted(pick))
+    return np.array(rows, dtype=np.int64)
+
+
+@pytest.mark.parametrize("layer", ["layer0", "layer1"])
+def test_blockscale_c5_shapes_quantised_on_the_gpu(layer):
+    """C5 at full size with the quantisation kernels feeding the GEMM: activations through the 1 x 128 kernel (its
+    permuted scale layout goes in as it is), weights through the 128 x 128 kernel.  layer0: gathered rows, K = 7168,
+    N = 2048; layer1: K = 2048, N = 7168 with the top-8 weight in the epilogue.  Sampled rows against the oracle on
+    the same bytes; and against the unquantised product (the quantisation error of e4m3 blocks, a few per cent)."""
+    from flux_amd import capi
+    wl = configs.make_workload("C5")
+    rng = np.random.default_rng(81)
+    e = wl.experts
+    if layer == "layer0":
+        a, w, kdim, ndim = wl.tensors["x"], wl.tensors["w1"], wl.hidden, wl.ffn
+        gather = torch.from_numpy(wl.gather_index).cuda()
+        row_w = None
+    else:
+        a, w, kdim, ndim = wl.tensors["act"], wl.tensors["w2"], wl.ffn, wl.hidden
+        gather = None
+        row_w = wl.row_weight
+    print(f"[case] blockscale C5 {layer} M={wl.rows} K={kdim} N={ndim}", flush=True)
+    qa_d, sa_d, _, _ = capi.quant_e4m3_block128(a.cuda())
+    qw_d, sw_d, _, _ = capi.quant_e4m3_square(w.cuda())
+    assert tuple(sa_d.shape) == ((a.shape[0] + 127) // 128, kdim // 128, 128) and tuple(sw_d.shape) == (e, ndim // 128, kdim // 128)
+    split_d = torch.from_numpy(wl.splits).cuda()
+    out = capi.grouped_gemm_blockscale(qa_d, qw_d, split_d, sa_d, sw_d, gather_a=gather,
+                                       row_scale=None if row_w is None else row_w.cuda())
+    assert tuple(out.shape) == (wl.rows, ndim)
+    qa, qw, sw = qa_d.cpu(), qw_d.cpu(), sw_d.cpu()
+    sa = sa_d.cpu().permute(0, 2, 1).reshape(-1, kdim // 128)[:a.shape[0]]      # back to [rows, K/128]
+    eor = routing.expert_of_row(wl.splits)
+    rows = sampled_rows(wl.splits, 6, rng)
+    num = den = num_u = 0.0
+    for ee in np.unique(eor[rows]):
+        r = rows[eor[rows] == ee]
+        src = torch.as_tensor(wl.gather_index[r] if gather is not None else r, dtype=torch.long)
+        ref = layers.fp8_blockscale_grouped_gemm_fp32(qa[src], sa[src], qw[int(ee):int(ee) + 1], sw[int(ee):int(ee) + 1],
+                                                      np.array([len(r)], dtype=np.int32))
+        unq = a[src].float() @ w[int(ee)].float().t()
+        if row_w is not None:
+            ref = ref * row_w[torch.as_tensor(r)][:, None]
+            unq = unq * row_w[torch.as_tensor(r)][:, None]
+        got = out[torch.as_tensor(r).cuda()].float().cpu()
+        num += float((got - ref).pow(2).sum())
+        num_u += float((got - unq).pow(2).sum())
+        den += float(ref.pow(2).sum())
+    assert (num / den) ** 0.5 < 3e-2
+    assert (num / den) ** 0.5 < 5e-3          # accumulation order and the bf16 rounding only
+    assert (num_u / den) ** 0.5 < 6e-2        # e4m3 block quantisation against the unquantised product

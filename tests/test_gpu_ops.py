@@ -321,3 +321,65 @@ def test_sm_margin_through_the_ops(c1):
     assert torch.equal(op0.forward(x, w1, sp, si, sm_margin=28), op0.forward(x, w1, sp, si))
     with pytest.raises(RuntimeError, match="sm_margin"):
         op0.forward(x, w1, sp, si, sm_margin=-1)
+
+
+def test_blockscale_gemm_op_dense_and_grouped():
+    """BlockScaleGemm.forward / forward_grouped (src/pybind/gemm_only.cc:77-139) fed by the Quantization op, the way
+    test/python/gemm_only/test_blockwise_scale_gemm_only.py drives them: both scale layouts of forward_grouped."""
+    g = torch.Generator().manual_seed(12)
+    experts, n, k = 3, 384, 512
+    split = np.array([200, 0, 313], dtype=np.int32)
+    m = int(split.sum())
+    x = torch.randn(m, k, generator=g).to(torch.bfloat16)
+    w = (torch.randn(experts, n, k, generator=g) * 0.05).to(torch.bfloat16)
+    q = flux_amd.Quantization(torch.bfloat16, torch.float8_e4m3fn)
+    qx, sx, _, _ = q.quantize_vector_blockwise(x.cuda(), return_tranpose=False)          # [ceil(M/128), K/128, 128]
+    qw, sw, _, _ = q.batch_quantize_square_blockwise(w.cuda(), return_tranpose=False)    # [E, N/128, K/128]
+    op = flux_amd.BlockScaleGemm(torch.float8_e4m3fn, torch.float8_e4m3fn, torch.bfloat16)
+    sa = sx.cpu().permute(0, 2, 1).reshape(-1, k // 128)[:m]
+    ref = layers.fp8_blockscale_grouped_gemm_fp32(qx.cpu(), sa, qw.cpu(), sw.cpu(), split)
+    out = op.forward_grouped(qx, torch.from_numpy(split), qw, input_scale=sx, weight_scale=sw)
+    assert out.dtype == torch.bfloat16
+    assert torch.allclose(out.float().cpu(), ref, rtol=1e-2, atol=1e-2 * float(ref.abs().max()))
+    # the reference's operand layouts: flat per-expert [K/128, M_e] and [K/128, N/128]
+    flat_a = layers.a_scale_to_expert_k_m(sa, split).cuda()
+    flat_b = sw.transpose(1, 2).contiguous().reshape(-1)
+    out2 = op.forward_grouped(qx, torch.from_numpy(split), qw, input_scale=flat_a, weight_scale=flat_b)
+    assert torch.equal(out2, out)
+    # dense
+    d = op.forward(qx, qw[0], input_scale=sx, weight_scale=sw[0].contiguous())
+    refd = layers.fp8_blockscale_grouped_gemm_fp32(qx.cpu(), sa, qw.cpu()[:1], sw.cpu()[:1], np.array([m], dtype=np.int32))
+    assert torch.allclose(d.float().cpu(), refd, rtol=1e-2, atol=1e-2 * float(refd.abs().max()))
+    with pytest.raises(RuntimeError, match="bias"):
+        op.forward(qx, qw[0], bias=torch.zeros(1, device="cuda"), input_scale=sx, weight_scale=sw[0].contiguous())
+    with pytest.raises(RuntimeError, match="cpu"):
+        op.forward_grouped(qx, torch.from_numpy(split).cuda(), qw, input_scale=sx, weight_scale=sw)
+
+
+def test_layer1_op_with_the_fused_epilogue_reduce(c1, monkeypatch):
+    """FLUX_AMD_LAYER1_REDUCE=fused: the layer1 op reduces in the GEMM's epilogue; same bound, and at top-2 the same
+    bits as the default two-pass form."""
+    wl = c1
+    t, k, e, h = wl.tokens, wl.topk, wl.experts, wl.hidden
+    act, w2 = wl.tensors["act"].cuda(), wl.tensors["w2"].cuda()
+    splits_cpu = torch.from_numpy(wl.splits)
+    idx = torch.from_numpy(wl.scatter_index.reshape(-1)).cuda()
+    ovs = wl.row_weight.cuda()
+    base = flux_amd.GemmGroupedV3GatherRS(e, t * k, h, k, 0, 1, 1, 1).forward_gather_rs(act, w2, splits_cpu, idx,
+                                                                                      output_vec_scale=ovs)
+    monkeypatch.setenv("FLUX_AMD_LAYER1_REDUCE", "fused")
+    op = flux_amd.GemmGroupedV3GatherRS(e, t * k, h, k, 0, 1, 1, 1)
+    monkeypatch.delenv("FLUX_AMD_LAYER1_REDUCE")
+    s_in, s_w = torch.tensor([0.75]), torch.rand(e) + 0.5
+    out = op.forward_gather_rs(act, w2, splits_cpu, idx, output_vec_scale=ovs)
+    ref = layers.layer1_fp32(wl.tensors["act"], wl.tensors["w2"], wl.splits, wl.scatter_index.reshape(-1), k,
+                             output_vec_scale=wl.row_weight)
+    close(out, ref)
+    assert torch.equal(out, base)
+    outs = op.forward_gather_rs(act, w2, splits_cpu, idx, input_scale=s_in.cuda(), weight_scale=s_w.cuda(),
+                                output_vec_scale=ovs)
+    close(outs, layers.layer1_fp32(wl.tensors["act"], wl.tensors["w2"], wl.splits, wl.scatter_index.reshape(-1), k,
+                                   s_in, s_w, wl.row_weight))
+    monkeypatch.setenv("FLUX_AMD_LAYER1_REDUCE", "sideways")
+    with pytest.raises(RuntimeError, match="FLUX_AMD_LAYER1_REDUCE"):
+        flux_amd.GemmGroupedV3GatherRS(e, t * k, h, k, 0, 1, 1, 1)

@@ -11,8 +11,8 @@ import flux_amd
 def test_module_exports_reference_names():
     m = flux_amd.flux_ths_pybind
     for name in ("MoeArguments", "DistEnvTPWithEP", "GemmGroupedV3AGScatter", "GemmGroupedV3GatherRS", "GemmGroupedV3",
-                 "Quantization", "calc_scatter_index", "topk_scatter_reduce", "bitwise_check", "init_flux_shm",
-                 "uniform_initialize", "load_tuning_record", "ProfilingContext", "TuningRecord"):
+                 "Quantization", "BlockScaleGemm", "calc_scatter_index", "topk_scatter_reduce", "bitwise_check",
+                 "init_flux_shm", "uniform_initialize", "load_tuning_record", "ProfilingContext", "TuningRecord"):
         assert hasattr(m, name), name
         assert getattr(flux_amd, name) is getattr(m, name)
     for cls, methods in ((m.GemmGroupedV3AGScatter, ("forward", "forward_multiple_weights", "clear_buffers", "profiling")),
@@ -20,6 +20,7 @@ def test_module_exports_reference_names():
                                                     "forward_gather_rs_no_zerobuffer", "ep_zero_buffer", "profiling")),
                          (m.ProfilingContext, ("get_code", "get_all_prof_results", "get_latest_prof_result",
                                                "get_latest_record", "get_all_records")),
+                         (m.BlockScaleGemm, ("forward", "forward_grouped")),
                          (m.Quantization, ("quantize_vector_blockwise", "quantize_square_blockwise",
                                            "batch_quantize_square_blockwise"))):
         for meth in methods:
@@ -37,6 +38,11 @@ def test_keyword_names_match_reference():
                "output_vec_scale", "fast_accum", "sm_margin", "with_stream_sync"):
         assert kw in doc, kw
     assert "return_tranpose" in m.Quantization.quantize_vector_blockwise.__doc__  # the reference's spelling
+    doc = m.BlockScaleGemm.forward_grouped.__doc__  # src/pybind/gemm_only.cc:130-139
+    for kw in ("input", "input_splits", "weight", "bias", "output", "input_scale", "weight_scale"):
+        assert kw in doc, kw
+    for kw in ("input_dtype", "weight_dtype", "output_dtype", "num_streams"):
+        assert kw in m.BlockScaleGemm.__init__.__doc__, kw
     doc = m.GemmGroupedV3GatherRS.__init__.__doc__
     for kw in ("total_num_experts", "max_m", "n_dim", "topk", "rank", "world_size", "tp_world_size", "ep_world_size",
                "max_input_groups", "ep_in_dp"):

@@ -154,3 +154,32 @@ def test_fp8_dequant_matmul_form():
     # e4m3 keeps 4 significant bits: ~3-5 % relative error against the unquantised product is inherent
     # (the benchmark's 3e-2 bound is against the dequantise-matmul itself); a wrong scale index gives O(1).
     assert 0 < err < 8e-2
+
+
+def test_blockscale_gemm_against_the_promotion_loop():
+    """The dequantise-by-block oracle against the promotion form written out as loops (float64): for every output
+    element, sum over K blocks of a_scale[r, kb] * w_scale[e, n // 128, kb] * (sum of the block's products).  A wrong
+    block index, a transposed scale or a scale applied per element instead of per block fails."""
+    g = torch.Generator().manual_seed(11)
+    rows, n, k, experts = 5, 130, 256, 2
+    split = np.array([2, 3], dtype=np.int32)
+    qa = torch.randn(rows, k, generator=g).to(torch.float8_e4m3fn)
+    qw = torch.randn(experts, n, k, generator=g).to(torch.float8_e4m3fn)
+    sa = torch.rand(rows, k // 128, generator=g) + 0.5
+    sw = torch.rand(experts, (n + 127) // 128, k // 128, generator=g) + 0.5
+    out = layers.fp8_blockscale_grouped_gemm_fp32(qa, sa, qw, sw, split)
+    eor = routing.expert_of_row(split)
+    ref = torch.zeros(rows, n, dtype=torch.float64)
+    for r in range(rows):
+        e = int(eor[r])
+        for col in range(n):
+            for kb in range(k // 128):
+                blk = slice(kb * 128, (kb + 1) * 128)
+                part = float((qa[r, blk].double() * qw[e, col, blk].double()).sum())
+                ref[r, col] += float(sa[r, kb]) * float(sw[e, col // 128, kb]) * part
+    assert torch.allclose(out.double(), ref, rtol=1e-5, atol=1e-5)
+    # layouts: the permuted 128-row form and the per-expert [K/128, M_e] form hold the same numbers
+    p128 = layers.a_scale_to_block128(sa)
+    assert tuple(p128.shape) == (1, 2, 128) and float(p128[0, 1, 3]) == float(sa[3, 1]) and float(p128[0, 0, 100]) == 0.0
+    ekm = layers.a_scale_to_expert_k_m(sa, split)
+    assert float(ekm[2 * 2 + 1 * 3 + 2]) == float(sa[4, 1])  # expert 1 starts at 2 rows * 2 blocks; block 1, its row 2
