@@ -148,7 +148,8 @@ __device__ __forceinline__ void store_tile(uint8_t *windows, const TileCtx &c, i
     // bf16 rows of whole tiles leave as whole 128-byte lines: two 32-column blocks per pass, packed to bf16
     // before the pass, so that the window (64 rows x 128 bytes) comes back as eight lanes x 16 bytes per row.
     // In 64-byte pieces a line is written in two halves at different times and part of the lines reach HBM
-    // twice.  Needs 16-byte aligned rows; other outputs take the 64-byte path below.
+    // twice.  Needs 16-byte aligned rows; other outputs take the 64-byte path below.  (The same form for the
+    // 32 x 32 blocks of the fp8 kernel measured 3-5 % slower than the 64-byte path on the fp8 benchmark shapes.)
     if ((n & 7) == 0 && (reinterpret_cast<uintptr_t>(d) & 15u) == 0) {
       uint8_t *const wlane = d + (static_cast<int64_t>(row_base + wrow0 + rr0) * n + wcol0 + cc * 8) * 2;
 #pragma unroll
@@ -338,9 +339,23 @@ struct TilePrefetch {
 // Ring fills address global memory through buffer resources: a scalar base per operand, a loop-invariant
 // 32-bit byte offset per lane and fill instruction, and the k offset as scalar offset.  Fill
 // instruction q of a tile covers rows [16q, 16q+16); tail rows re-read the last valid row.
+// The rows of A this lane's X fill instructions of tile t fetch (tail rows repeat the last valid row): the
+// gather indices when A is gathered.  Split from setup_operands so that a tile can request the indices of the
+// tile after it before its own main loop, and find them in registers when it sets that tile up.
+template <int XL>
+__device__ __forceinline__ void load_gather_rows(const GemmParams &p, const TileCtx &c, const TileDesc &t, int (&arow)[XL]) {
+#pragma unroll
+  for (int j = 0; j < XL; ++j) {
+    int xr = t.m0 + (XL * c.wave + j) * 16 + c.fill_row;
+    if (xr > t.rows_e - 1) xr = t.rows_e - 1;
+    if (xr < 0) xr = 0;
+    arow[j] = p.gather_a[t.row_base + xr];
+  }
+}
+
 template <int XL, int WL>
 __device__ __forceinline__ void setup_operands(const GemmParams &p, const TileCtx &c, const TileDesc &t,
-                                               TileOperands<XL, WL> &op) {
+                                               TileOperands<XL, WL> &op, const int *preloaded_rows = nullptr) {
   const bool gathered = p.gather_a != nullptr;
   const uint8_t *xbase = gathered ? p.a : p.a + static_cast<int64_t>(t.row_base + t.m0) * c.kbytes;
   const int64_t xrows = gathered ? p.a_rows : t.rows_e - t.m0;
@@ -354,7 +369,7 @@ __device__ __forceinline__ void setup_operands(const GemmParams &p, const TileCt
     if (xr > t.rows_e - 1) xr = t.rows_e - 1;
     int64_t arow = xr - t.m0;
     if (gathered) {
-      arow = p.gather_a[t.row_base + xr];
+      arow = preloaded_rows ? preloaded_rows[j] : p.gather_a[t.row_base + xr];
       if (p.a_rows > 0) arow = arow < 0 ? 0 : (arow >= p.a_rows ? p.a_rows - 1 : arow);
     }
     op.xoff[j] = static_cast<uint32_t>(arow * c.kbytes) + c.fill_chunk * 16;
@@ -410,6 +425,27 @@ __device__ __forceinline__ void fill_any(const TileOperands<XL, WL> &op, uint8_t
 // Requests the first LA k-steps of a tile pair by pair into ring slots 0..LA-1 (q is a constant after unrolling).
 template <int XL, int WL>
 __device__ __forceinline__ void issue_first_pairs(const TileOperands<XL, WL> &op, uint8_t *smem, const TileCtx &c) {
+  if (c.nkf >= Ring<XL, WL>::LA) {
+    // All of these k-steps are whole ones (every K of practical interest): the same fills without the per-fill
+    // choice between operand, partial step and zero page; slots and k offsets are immediates.
+#pragma unroll
+    for (int s = 0; s < Ring<XL, WL>::LA; s += 2) {
+#pragma unroll
+      for (int q = 0; q < XL + WL; ++q) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          if (q < XL)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(op.xrsrc, (lds_ptr_t)(smem + (s + h) * Ring<XL, WL>::SB + (XL * c.wave + q) * 1024),
+                                                     16, static_cast<int>(op.xoff[q < XL ? q : 0]), (s + h) * KBYTES, 0, 0);
+          else
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                op.wrsrc, (lds_ptr_t)(smem + (s + h) * Ring<XL, WL>::SB + Ring<XL, WL>::XB + (WL * c.wave + (q - XL)) * 1024), 16,
+                static_cast<int>(op.woff[q >= XL ? q - XL : 0]), (s + h) * KBYTES, 0, 0);
+        }
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int s = 0; s < Ring<XL, WL>::LA; s += 2) {
 #pragma unroll
@@ -461,6 +497,11 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
     }
   }
   if (!prefetched) setup_operands<XLOADS, WLOADS>(p, c, t, op);
+  // The gather indices of the next tile (when it is a whole macro tile, whose first fills this tile requests
+  // ahead of its epilogue): requested now, so that their latency passes under this tile's main loop.
+  int next_rows[4] = {0, 0, 0, 0};
+  const bool preload_next = next.kind == 0 && p.gather_a != nullptr;
+  if (preload_next) load_gather_rows<4>(p, c, next, next_rows);
   const __amdgpu_buffer_rsrc_t xrsrc = op.xrsrc, wrsrc = op.wrsrc;
   const __amdgpu_buffer_rsrc_t zrsrc = make_rsrc(g_zero_page, 1024);
   const uint32_t zoff = lane * 16;
@@ -494,9 +535,12 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
   auto fill_m0 = [&](auto SLOT, auto Q) {
     constexpr int slot = decltype(SLOT)::value, q = decltype(Q)::value;
     const uint32_t dst = q < XLOADS ? xdst32 + slot * SB + q * 1024 : wdst32 + slot * SB + (q - XLOADS) * 1024;
-    // M0 is declared clobbered so that the compiler never assumes a value it wrote to M0 earlier (for a fill it
-    // emitted itself) is still there after this statement.
-    asm volatile("s_mov_b32 m0, %0" : : "s"(dst) : "memory", "m0");
+    // M0 cannot be named in the clobber list (the compiler reserves it and warns that such a clobber is not
+    // honoured), so nothing tells the compiler that M0 changes here.  It is safe while the compiler itself puts
+    // no M0 use between this statement and the load that follows it (the schedule barriers around every MFMA slot
+    // see to that) and re-initialises M0 before every fill it emits itself (it does: the builtin writes M0 each
+    // time); the test that compares this variant bit for bit with the builtin-only fills guards both.
+    asm volatile("s_mov_b32 m0, %0" : : "s"(dst) : "memory");
   };
   auto fill_go = [&](auto Q, int kbyte) {
     constexpr int q = decltype(Q)::value;
@@ -778,7 +822,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
   // epilogue's LDS windows lie in slot 4.
   pf.valid = false;
   if (next.kind == 0) {
-    setup_operands<4, 4>(p, c, next, pf.op);
+    setup_operands<4, 4>(p, c, next, pf.op, preload_next ? next_rows : nullptr);
     issue_first_pairs<4, 4>(pf.op, smem, c);
     pf.valid = true;
   }
