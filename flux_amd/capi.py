@@ -9,7 +9,9 @@ import os
 
 import torch
 
-_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libfluxmi_kernels.so")
+# $FLUX_AMD_KERNEL_LIB names another build of the same library (an A/B comparison, a debug build).
+_LIB_PATH = os.environ.get("FLUX_AMD_KERNEL_LIB") or os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib",
+                                                                  "libfluxmi_kernels.so")
 _lib = None
 
 BF16 = 0

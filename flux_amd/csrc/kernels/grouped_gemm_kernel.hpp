@@ -632,21 +632,36 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
                                              static_cast<int>(in ? as_voff : static_cast<uint32_t>(lane * 4)),
                                              in ? kb * as_kstep : 0, 0, 0);
   };
-  // End of a pair of k-steps: main += acc * (row scale * block scale of B), acc = 0.
-  auto promote = [&](int slot, int kb) {
+  // The block scale of B for scale block kb: one value per pair of k-steps, fetched with a scalar load when the
+  // pair starts (through the constant address space: as a vector load it would sit in the queue of the ring fills,
+  // and waiting for it would drain them all) and used when the pair ends.
+  typedef const __attribute__((address_space(4))) float *ConstF32;
+  float bsv = 0.f;
+  auto bscale_load = [&](int kb) {
     if constexpr (BS) {
-      const float bsv = kernel_args()->b_scale[__builtin_amdgcn_readfirstlane(bs_base + kb * bs_kstep)];
+      const ConstF32 bs = (ConstF32)(kernel_args()->b_scale);
+      bsv = bs[__builtin_amdgcn_readfirstlane(bs_base + (kb < kblocks ? kb : 0) * bs_kstep)];
+    }
+  };
+  // Promotion of a pair of k-steps: main += acc * (row scale * block scale of B), acc = 0, block by block during the
+  // pair's second step: block b is promoted two MFMA slots after its last MFMA was issued, in the shadow of the
+  // MFMAs of the blocks after it; the last two blocks follow the step.
+  constexpr int PROMOTE_LAG = 2;
+  float psc[BS ? MBK : 1];
+  auto promote_begin = [&](int slot) {
+    if constexpr (BS) {
       const float *srow = reinterpret_cast<const float *>(smem + slot * SB + SCALE_OFF) + wm * (32 * MB) + (lane & 31);
 #pragma unroll
-      for (int i = 0; i < MBK; ++i) {
-        const float sc = srow[i * 32] * bsv;
+      for (int i = 0; i < MBK; ++i) psc[i] = srow[i * 32] * bsv;
+    }
+  };
+  auto promote_block = [&](auto B) {
+    if constexpr (BS) {
+      constexpr int b = decltype(B)::value, i = b / NBK, j = b % NBK;
 #pragma unroll
-        for (int j = 0; j < NBK; ++j)
-#pragma unroll
-          for (int v = 0; v < Geom<ELT>::NACC; ++v) {
-            main_acc[i][j][v] = fmaf(acc[i][j][v], sc, main_acc[i][j][v]);
-            acc[i][j][v] = 0.f;
-          }
+      for (int v = 0; v < Geom<ELT>::NACC; ++v) {
+        main_acc[i][j][v] = fmaf(acc[i][j][v], psc[i], main_acc[i][j][v]);
+        acc[i][j][v] = 0.f;
       }
     }
   };
@@ -697,7 +712,10 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
     }
     __builtin_amdgcn_s_barrier();     // ... for every wave's share; and everybody is done reading stage u
     __builtin_amdgcn_sched_barrier(0);
-    if constexpr (BS && even) scale_fill((e0 + LA) % STG, (kbase / KBYTES + e0 + LA) >> 1);
+    if constexpr (BS && even) {
+      scale_fill((e0 + LA) % STG, (kbase / KBYTES + e0 + LA) >> 1);
+      bscale_load((kbase / KBYTES + e0) >> 1);
+    }
     static_for<0, NM>([&](auto T) {
       constexpr int t = decltype(T)::value;
       static_for<0, NR>([&](auto R) {
@@ -723,10 +741,14 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
         if constexpr (at % NM != 0 && at - 1 == t + (even ? 0 : NM))
           fill_m0(std::integral_constant<int, (e0 + LA + (d & 1)) % STG>{}, std::integral_constant<int, (d >> 1)>{});
       });
+      if constexpr (BS && !even && t == 0) promote_begin(e0 % STG);
       mfma_slot<ELT, MBK, NBK>(t, xc, wc, acc);
+      if constexpr (BS && !even && t >= PROMOTE_LAG) promote_block(std::integral_constant<int, (t >= PROMOTE_LAG ? t - PROMOTE_LAG : 0)>{});
       __builtin_amdgcn_sched_barrier(0);
     });
-    if constexpr (BS && !even) promote(e0 % STG, (kbase / KBYTES + e0) >> 1);
+    if constexpr (BS && !even) {
+      static_for<NM - PROMOTE_LAG, NM>([&](auto B) { promote_block(B); });
+    }
     FLUXMI_WAITCNT(63, 0);  // the fragments of the next step are in registers (requested long ago)
     __builtin_amdgcn_sched_barrier(0);
   };
@@ -743,7 +765,10 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
     const int e0 = even ? ks : ks - 1;
     const int rslot = (ks + 1) % STG, pslot0 = (e0 + LA) % STG, pslot1 = (e0 + LA + 1) % STG;
     if constexpr (BS) {
-      if (even) scale_fill(pslot0, (e0 + LA) >> 1);
+      if (even) {
+        scale_fill(pslot0, (e0 + LA) >> 1);
+        bscale_load(e0 >> 1);
+      }
     }
     static_for<0, NM>([&](auto T) {
       constexpr int t = decltype(T)::value;
@@ -760,11 +785,17 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
           if (at - NM == t && !even) fill_dyn((d & 1) ? pslot1 : pslot0, std::integral_constant<int, (d >> 1)>{}, e0 + LA + (d & 1));
         }
       });
+      if constexpr (BS && t == 0) {
+        if (!even) promote_begin(e0 % STG);
+      }
       mfma_slot<ELT, MBK, NBK>(t, xc, wc, acc);
+      if constexpr (BS && t >= PROMOTE_LAG) {
+        if (!even) promote_block(std::integral_constant<int, (t >= PROMOTE_LAG ? t - PROMOTE_LAG : 0)>{});
+      }
       __builtin_amdgcn_sched_barrier(0);
     });
     if constexpr (BS) {
-      if (!even) promote(e0 % STG, e0 >> 1);
+      if (!even) static_for<NM - PROMOTE_LAG, NM>([&](auto B) { promote_block(B); });
     }
     FLUXMI_WAITCNT(63, 0);
     __builtin_amdgcn_sched_barrier(0);
