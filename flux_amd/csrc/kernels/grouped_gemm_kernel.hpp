@@ -107,9 +107,18 @@ __device__ __forceinline__ float acc_read(float a) {
   return v;
 }
 
+// Compile-time loop: f(integral_constant<int, I>) for I in [0, N).
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F &&f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<I + 1, N>(f);
+  }
+}
+
 // Epilogue of one wave: acc (32*MB rows x 32*NB columns, MFMA layout) -> scaled, cast, stored.
-// Blocks of 64 rows x 32 columns go through one of two 8 KiB LDS windows in fp32 (alternating, so the
-// writes of a block do not wait for the reads of the one before) and come back with eight lanes per
+// Blocks of 32 rows x 32 columns go through the two 4 KiB halves of the wave's LDS window in fp32 (alternating, so
+// the writes of a block do not wait for the reads of the one before) and come back with eight lanes per
 // row (j below counts 32-column groups, ip 64-row groups).  FULL: every row and column of the wave's quarter exists and rows are stored where they are (no
 // scatter), so no store is predicated.  OUT_F32 selects the output element type.  !SCALED: every scale
 // factor is 1 and the multiplications are left out.
@@ -196,89 +205,103 @@ __device__ __forceinline__ void store_tile(uint8_t *windows, const TileCtx &c, i
       return;
     }
   }
-  int block = 0;
+  // 64-byte (bf16) / 128-byte (fp32) pieces: passes of 32 rows x 32 columns through the two 4 KiB halves of the
+  // window in fp32, software-pipelined: while the rows of pass p come back from LDS and are stored, the
+  // accumulators of pass p + 1 are already being written to the other half, so that the LDS round trip of a pass
+  // is not exposed.  Pass p = ((j * (MB / 2) + ip) * 2 + hh): column group j, 64-row group ip, its 32-row half hh.
+  constexpr int NPASS = NB * (MB / 2) * 2;
+  float4 csj[NB];  // column scales of this lane's 4-column chunk in every column group
 #pragma unroll
   for (int j = 0; j < NB; ++j) {
     const int col = wcol0 + j * 32 + cc * 4;
-    float4 cs = make_float4(1.f, 1.f, 1.f, 1.f);
-    if (col_scale && (FULL || col < n)) cs = *reinterpret_cast<const float4 *>(col_scale + static_cast<int64_t>(e) * n + col);
+    csj[j] = make_float4(1.f, 1.f, 1.f, 1.f);
+    if (col_scale && (FULL || col < n)) csj[j] = *reinterpret_cast<const float4 *>(col_scale + static_cast<int64_t>(e) * n + col);
+  }
+  // A lane holds one row of a block and groups of 4 consecutive columns of it: with 16x16 blocks one group,
+  // columns 4 * (lane / 16); with 32x32 blocks four, columns 8q + 4 * (lane / 32).
+  auto write_half = [&](auto PC) {
+    constexpr int ps = decltype(PC)::value, hh = ps & 1, blk = ps >> 1, ip = blk % (MB / 2), j = blk / (MB / 2);
+    uint8_t *half = windows + hh * 4096;
 #pragma unroll
-    for (int ip = 0; ip < MB / 2; ++ip, ++block) {
-      uint8_t *window = windows;
-      // write phase.  A lane holds one row of a block and groups of 4 consecutive columns of it: with
-      // 16x16 blocks one group, columns 4 * (lane / 16); with 32x32 blocks four, columns 8q + 4 * (lane / 32).
+    for (int i2 = 0; i2 < 32 / BLK; ++i2) {
+      const int i = ip * (64 / BLK) + hh * (32 / BLK) + i2;
+      const int r = i2 * BLK + (lane & (BLK - 1));
 #pragma unroll
-      for (int ii = 0; ii < 64 / BLK; ++ii) {
-        const int i = ip * (64 / BLK) + ii;
-        const int r = ii * BLK + (lane & (BLK - 1));
+      for (int jj = 0; jj < 32 / BLK; ++jj) {
+        const int jb = j * (32 / BLK) + jj;
 #pragma unroll
-        for (int jj = 0; jj < 32 / BLK; ++jj) {
-          const int jb = j * (32 / BLK) + jj;
-#pragma unroll
-          for (int q = 0; q < Geom<ELT>::NACC / 4; ++q) {
-            const int chunk = BLK == 32 ? 2 * q + h : jj * 4 + (lane >> 4);
-            float4 v = make_float4(acc_read(acc[i][jb][4 * q + 0]), acc_read(acc[i][jb][4 * q + 1]),
-                                   acc_read(acc[i][jb][4 * q + 2]), acc_read(acc[i][jb][4 * q + 3]));
-            if constexpr (SCALED) v = make_float4(v.x * rs[i], v.y * rs[i], v.z * rs[i], v.w * rs[i]);
-            *reinterpret_cast<float4 *>(window + r * 128 + ((chunk ^ ((r >> 1) & 7)) << 4)) = v;
-          }
-        }
-      }
-      // store phase: 8 lanes per row, 8 rows per instruction
-      float4 v[8];
-#pragma unroll
-      for (int it = 0; it < 8; ++it) {
-        const int rr = it * 8 + rr0;
-        v[it] = *reinterpret_cast<const float4 *>(window + rr * 128 + ((cc ^ ((rr >> 1) & 7)) << 4));
-      }
-      uint8_t *dp = dlane + (static_cast<int64_t>(ip) * 8) * rowgroup_bytes + j * 32 * ELT_OUT;
-#pragma unroll
-      for (int it = 0; it < 8; ++it, dp += rowgroup_bytes) {
-        uint8_t *dst = dp;
-        if constexpr (!FULL) {
-          const int m = wrow0 + ip * 64 + it * 8 + rr0;
-          if (m >= rows_e || col >= n) continue;  // n % 4 == 0: a chunk is all in or all out
-          if (scatter) {
-            const int64_t drow = scatter[row_base + m];
-            if (drow < 0 || drow >= d_rows) continue;
-            dst = d + (drow * n + col) * ELT_OUT;
-          }
-        }
-        float4 o = v[it];
-        if constexpr (SCALED) o = make_float4(o.x * cs.x, o.y * cs.y, o.z * cs.z, o.w * cs.w);
-        if constexpr (OUT_F32) {
-          if (accumulate) {
-            // Hardware fp32 atomic adds without return: sorted rows of one token meet in that token's row of D.
-            float *df = reinterpret_cast<float *>(dst);
-            unsafeAtomicAdd(df + 0, o.x);
-            unsafeAtomicAdd(df + 1, o.y);
-            unsafeAtomicAdd(df + 2, o.z);
-            unsafeAtomicAdd(df + 3, o.w);
-          } else if (nt_stores) {
-            typedef float f32x4_t __attribute__((ext_vector_type(4)));
-            const f32x4_t ov = {o.x, o.y, o.z, o.w};
-            __builtin_nontemporal_store(ov, reinterpret_cast<f32x4_t *>(dst));
-          } else {
-            *reinterpret_cast<float4 *>(dst) = o;
-          }
-        } else {
-          u32x2 b;
-          b[0] = pack_bf16x2(o.x, o.y);
-          b[1] = pack_bf16x2(o.z, o.w);
-          *reinterpret_cast<u32x2 *>(dst) = b;
+        for (int q = 0; q < Geom<ELT>::NACC / 4; ++q) {
+          const int chunk = BLK == 32 ? 2 * q + h : jj * 4 + (lane >> 4);
+          float4 v = make_float4(acc_read(acc[i][jb][4 * q + 0]), acc_read(acc[i][jb][4 * q + 1]),
+                                 acc_read(acc[i][jb][4 * q + 2]), acc_read(acc[i][jb][4 * q + 3]));
+          if constexpr (SCALED) v = make_float4(v.x * rs[i], v.y * rs[i], v.z * rs[i], v.w * rs[i]);
+          *reinterpret_cast<float4 *>(half + r * 128 + ((chunk ^ ((r >> 1) & 7)) << 4)) = v;
         }
       }
     }
-  }
-}
-
-// Compile-time loop: f(integral_constant<int, I>) for I in [0, N).
-template <int I, int N, class F>
-__device__ __forceinline__ void static_for(F &&f) {
-  if constexpr (I < N) {
-    f(std::integral_constant<int, I>{});
-    static_for<I + 1, N>(f);
-  }
+  };
+  // 8 lanes per row, 8 rows per instruction
+  auto read_half = [&](auto PC, float4 (&v)[4]) {
+    constexpr int hh = decltype(PC)::value & 1;
+    const uint8_t *half = windows + hh * 4096;
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+      const int rr = it * 8 + rr0;
+      v[it] = *reinterpret_cast<const float4 *>(half + rr * 128 + ((cc ^ ((rr >> 1) & 7)) << 4));
+    }
+  };
+  auto store_half = [&](auto PC, const float4 (&v)[4]) {
+    constexpr int ps = decltype(PC)::value, hh = ps & 1, blk = ps >> 1, ip = blk % (MB / 2), j = blk / (MB / 2);
+    const int col = wcol0 + j * 32 + cc * 4;
+    const float4 cs = csj[j];
+    uint8_t *dp = dlane + (static_cast<int64_t>(ip) * 8 + hh * 4) * rowgroup_bytes + j * 32 * ELT_OUT;
+#pragma unroll
+    for (int it = 0; it < 4; ++it, dp += rowgroup_bytes) {
+      uint8_t *dst = dp;
+      if constexpr (!FULL) {
+        const int m = wrow0 + ip * 64 + hh * 32 + it * 8 + rr0;
+        if (m >= rows_e || col >= n) continue;  // n % 4 == 0: a chunk is all in or all out
+        if (scatter) {
+          const int64_t drow = scatter[row_base + m];
+          if (drow < 0 || drow >= d_rows) continue;
+          dst = d + (drow * n + col) * ELT_OUT;
+        }
+      }
+      float4 o = v[it];
+      if constexpr (SCALED) o = make_float4(o.x * cs.x, o.y * cs.y, o.z * cs.z, o.w * cs.w);
+      if constexpr (OUT_F32) {
+        if (accumulate) {
+          // Hardware fp32 atomic adds without return: sorted rows of one token meet in that token's row of D.
+          float *df = reinterpret_cast<float *>(dst);
+          unsafeAtomicAdd(df + 0, o.x);
+          unsafeAtomicAdd(df + 1, o.y);
+          unsafeAtomicAdd(df + 2, o.z);
+          unsafeAtomicAdd(df + 3, o.w);
+        } else if (nt_stores) {
+          typedef float f32x4_t __attribute__((ext_vector_type(4)));
+          const f32x4_t ov = {o.x, o.y, o.z, o.w};
+          __builtin_nontemporal_store(ov, reinterpret_cast<f32x4_t *>(dst));
+        } else {
+          *reinterpret_cast<float4 *>(dst) = o;
+        }
+      } else {
+        u32x2 b;
+        b[0] = pack_bf16x2(o.x, o.y);
+        b[1] = pack_bf16x2(o.z, o.w);
+        *reinterpret_cast<u32x2 *>(dst) = b;
+      }
+    }
+  };
+  float4 va[4], vb[4];
+  write_half(std::integral_constant<int, 0>{});
+  static_for<0, NPASS>([&](auto PC) {
+    constexpr int ps = decltype(PC)::value;
+    if constexpr ((ps & 1) == 0) read_half(PC, va);
+    else read_half(PC, vb);
+    if constexpr (ps + 1 < NPASS) write_half(std::integral_constant<int, (ps + 1 < NPASS ? ps + 1 : 0)>{});
+    if constexpr ((ps & 1) == 0) store_half(PC, va);
+    else store_half(PC, vb);
+  });
 }
 
 // Buffer resource over [base, base + bytes): loads past the end return zero instead of faulting.

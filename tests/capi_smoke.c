@@ -92,6 +92,23 @@ int main(void) {
       fprintf(stderr, "routing: gather_index / topk_index are not the inverse permutation at %d\n", i);
       return 1;
     }
+  /* the same sort over the library's static scratch array: the entry point that allocates nothing */
+  {
+    static int32_t scatter2[M], gather2[M], splits2[E];
+    HIP_OK(hipMemset(d_scatter, 0xff, sizeof scatter));
+    HIP_OK(hipMemset(d_gather, 0xff, sizeof gather));
+    HIP_OK(hipMemset(d_splits, 0xff, sizeof splits));
+    FLUX_OK(fluxmi_moe_route_sort_static(d_choosed, T, TOPK, E, d_splits, d_offsets, d_scatter, d_gather, d_tki, NULL));
+    HIP_OK(hipDeviceSynchronize());
+    HIP_OK(hipMemcpy(splits2, d_splits, sizeof splits2, hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(scatter2, d_scatter, sizeof scatter2, hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(gather2, d_gather, sizeof gather2, hipMemcpyDeviceToHost));
+    if (memcmp(splits2, splits, sizeof splits) || memcmp(scatter2, scatter, sizeof scatter) ||
+        memcmp(gather2, gather, sizeof gather) || fluxmi_moe_route_sort_static_max_bytes() < ws_bytes) {
+      fprintf(stderr, "routing: the static-scratch sort differs from the workspace sort\n");
+      return 1;
+    }
+  }
   printf("routing ok\n");
 
   /* ---- layer0: gather + grouped GEMM, bf16 ------------------------------------------------------ */
@@ -118,6 +135,10 @@ int main(void) {
   ga.splits = d_splits;
   ga.gather_a = d_gather;
   ga.scalar_scale = 1.0f;
+  if (fluxmi_grouped_gemm_kernel_kind(&ga) != 1) {
+    fprintf(stderr, "grouped GEMM: K = %d bf16 (rows of %d bytes) must take the MFMA kernel\n", H, 2 * H);
+    return 1;
+  }
   FLUX_OK(fluxmi_grouped_gemm(&ga, NULL, 0, NULL));
   HIP_OK(hipDeviceSynchronize());
   HIP_OK(hipMemcpy(y, d_y, sizeof y, hipMemcpyDeviceToHost));
@@ -161,6 +182,39 @@ int main(void) {
       }
     }
   printf("gather-reduce ok\n");
+
+  /* ---- the same layer with the reduction in the GEMM's epilogue: out2[t] = sum_j w[r_j] * (x[t] @ W[e_j]^T) ---- */
+  {
+    static uint16_t out2[T * N];
+    uint16_t *d_out2;
+    void *d_acc;
+    const size_t acc_bytes = fluxmi_grouped_gemm_topk_reduce_workspace_bytes(T, N);
+    HIP_OK(hipMalloc((void **)&d_out2, sizeof out2));
+    HIP_OK(hipMalloc(&d_acc, acc_bytes));
+    fluxmi_grouped_gemm_args fa = ga;
+    fa.d = NULL;
+    fa.row_scale = d_row_w;
+    FLUX_OK(fluxmi_grouped_gemm_topk_reduce(&fa, d_gather, T, d_out2, d_acc, acc_bytes, NULL));
+    HIP_OK(hipDeviceSynchronize());
+    HIP_OK(hipMemcpy(out2, d_out2, sizeof out2, hipMemcpyDeviceToHost));
+    for (int t = 0; t < T; ++t)
+      for (int n = 0; n < N; ++n) {
+        float want = 0.f;
+        for (int j = 0; j < TOPK; ++j) {
+          const int r = scatter[t * TOPK + j];
+          int e = 0;
+          while (r >= offsets[e] + splits[e]) ++e;
+          float acc = 0.f;
+          for (int k = 0; k < H; ++k) acc += bf2f(x[t * H + k]) * bf2f(w[(e * N + n) * H + k]);
+          want += row_w[r] * acc;
+        }
+        if (fabsf(bf2f(out2[t * N + n]) - want) > 1e-2f + 1e-2f * fabsf(want)) {
+          fprintf(stderr, "fused reduce: token %d col %d got %g want %g\n", t, n, bf2f(out2[t * N + n]), want);
+          return 1;
+        }
+      }
+    printf("fused epilogue reduce ok\n");
+  }
 
   /* ---- e4m3 quantisation per row: scale_inv = amax / 448, the row's largest element maps to +-448 ------- */
   static uint8_t q[T * H];
