@@ -76,18 +76,23 @@ class Events:
         return {"mean": sum(v) / len(v), "median": statistics.median(v), "min": min(v)}
 
 
-def time_loop(torch, fn, iters, warm=3):
+def time_loop(torch, fn, iters, warm=5, reps=3):
+    """Mean time of one call in ms: the median over `reps` back-to-back loops of `iters` calls.  The first loop after
+    a change of kernel runs while the board settles to the new kernel's power draw and can read 10-20 % off."""
     for _ in range(warm):
         fn()
     torch.cuda.synchronize()
-    e0 = torch.cuda.Event(enable_timing=True)
-    e1 = torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(iters):
-        fn()
-    e1.record()
-    torch.cuda.synchronize()
-    return e0.elapsed_time(e1) / iters
+    means = []
+    for _ in range(reps):
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        means.append(e0.elapsed_time(e1) / iters)
+    return statistics.median(means)
 
 
 class ClockSampler(threading.Thread):
@@ -302,6 +307,23 @@ def aux_measurements(torch, capi, configs, a, wl, dev, gen, tensors):
         sb = torch.rand(e5, n5 // 128, k5 // 128, generator=gen, device=dev) + 0.5
         t_bs = time_loop(torch, lambda: capi.grouped_gemm_blockscale(a8, b8, sp5, sa, sb, out=d5), 20)
         kernels[f"gemm_fp8_blockscale_c5_{tag}"] = gemm_entry(t_bs, f5, PEAK_FP8_TFLOPS, "frac_fp8_peak")
+        # The library's fp8 GEMM (torch._scaled_mm = hipBLASLt) for scale: the same work as a loop of per-expert
+        # GEMMs, and one dense GEMM of the same FLOPs with a single weight matrix (1/32 of the weight bytes).
+        try:
+            one = torch.ones((), device=dev)
+            rows5 = m5 // e5
+
+            def lib8_loop():
+                for ei in range(e5):
+                    torch._scaled_mm(a8[ei * rows5:(ei + 1) * rows5], b8[ei].t(), scale_a=one, scale_b=one,
+                                     out_dtype=torch.bfloat16, out=d5[ei * rows5:(ei + 1) * rows5])
+
+            kernels[f"library_fp8_gemm_loop_c5_{tag}"] = gemm_entry(time_loop(torch, lib8_loop, 10), f5, PEAK_FP8_TFLOPS, "frac_fp8_peak")
+            t_dense = time_loop(torch, lambda: torch._scaled_mm(a8, b8[0].t(), scale_a=one, scale_b=one,
+                                                                 out_dtype=torch.bfloat16, out=d5), 20)
+            kernels[f"library_fp8_gemm_dense_one_weight_c5_{tag}"] = gemm_entry(t_dense, f5, PEAK_FP8_TFLOPS, "frac_fp8_peak")
+        except Exception as ex:  # the library may not offer this dtype / layout
+            kernels[f"library_fp8_gemm_loop_c5_{tag}"] = {"error": repr(ex)[:120]}
         del a8, b8, d5, cs5, sa, sb
 
     # -- the same two C3 GEMMs as a loop of library GEMMs (torch.mm = hipBLASLt), one per expert, on rows that
