@@ -199,6 +199,59 @@ torch::Tensor BlockScaleGemm::forward_grouped(torch::Tensor input, torch::Tensor
   return blockscale_run(input, weight, input_splits, output, input_scale, a_layout, weight_scale, b_layout, output_dtype_);
 }
 
+// The reference runs this form as one GEMM per expert spread over its streams (blockscale_gemm.cc:376-486); here it
+// is the same single launch as forward_grouped.  input_scale is [M, K/128] with any strides (the reference's callers
+// pass the transposed view of a [K/128, M] tensor, :440-447), weight_scale [E, N/128, K/128].
+torch::Tensor BlockScaleGemm::forward_multistream(torch::Tensor input, torch::Tensor input_splits, torch::Tensor weight,
+                                                  std::optional<torch::Tensor> bias, std::optional<torch::Tensor> output,
+                                                  std::optional<torch::Tensor> input_scale,
+                                                  std::optional<torch::Tensor> weight_scale) {
+  TORCH_CHECK(!bias.has_value(), "BlockScaleGemm: bias is not supported");
+  TORCH_CHECK(input_scale.has_value(), "cur_input_scale is required but missing!");
+  TORCH_CHECK(weight_scale.has_value(), "BlockScaleGemm: weight_scale is required");
+  FLUX_AMD_CHECK_INPUT(input, input_dtype_);
+  FLUX_AMD_CHECK_INPUT(weight, weight_dtype_);
+  FLUX_AMD_CHECK_NDIM(input, 2);
+  FLUX_AMD_CHECK_NDIM(weight, 3);
+  FLUX_AMD_CHECK_NDIM(input_splits, 1);
+  FLUX_AMD_CHECK_NDIM((*input_scale), 2);
+  FLUX_AMD_CHECK_NDIM((*weight_scale), 3);
+  TORCH_CHECK(!input_splits.is_cuda(), "input splits is not on cpu");
+  TORCH_CHECK(input_splits.size(0) == weight.size(0), "splits 0-dim mismatch: ", input_splits.size(0), " != ",
+              weight.size(0));
+  TORCH_CHECK(input_splits.sum().item<int64_t>() <= input.size(0), "input_splits sum exceeds the rows of input");
+  const int64_t m = input.size(0), kb = input.size(1) / kBlock;
+  TORCH_CHECK(input_scale->is_cuda() && input_scale->scalar_type() == at::kFloat && input_scale->size(0) == m &&
+                  input_scale->size(1) == kb,
+              "input_scale must be a float32 device tensor of shape [", m, ", ", kb, "]");
+  // [M, K/128] -> [ceil(M/128), K/128, 128], the layout the kernel reads rows of scales from.
+  const int64_t mb = (m + kBlock - 1) / kBlock;
+  torch::Tensor padded = torch::zeros({mb * kBlock, kb}, input_scale->options());
+  padded.narrow(0, 0, m).copy_(*input_scale);
+  torch::Tensor blocked = padded.view({mb, kBlock, kb}).permute({0, 2, 1}).contiguous();
+  return blockscale_run(input, weight, input_splits, output, blocked, FLUXMI_ASCALE_BLOCK128, weight_scale->contiguous(),
+                        FLUXMI_BSCALE_N_K, output_dtype_);
+}
+
+// The reference's second implementation of forward (blockscale_gemm.cc:954-973); one kernel serves both here.  Its
+// per-column form of the weight scales is not built.
+torch::Tensor BlockScaleGemm::reference(torch::Tensor input, torch::Tensor weight, std::optional<torch::Tensor> bias,
+                                        std::optional<torch::Tensor> output, std::optional<torch::Tensor> input_scale,
+                                        std::optional<torch::Tensor> weight_scale, bool is_groupwise_b) {
+  TORCH_CHECK(!is_groupwise_b, "BlockScaleGemm.reference: per-column weight scales (is_groupwise_b) are not supported");
+  return forward(std::move(input), std::move(weight), std::move(bias), std::move(output), std::move(input_scale),
+                 std::move(weight_scale));
+}
+
+// The reference times every registered kernel configuration and runs the best (blockscale_gemm.cc:975-1023); there is
+// one configuration here, so this is forward.
+torch::Tensor BlockScaleGemm::profiling(torch::Tensor input, torch::Tensor weight, std::optional<torch::Tensor> bias,
+                                        std::optional<torch::Tensor> output, std::optional<torch::Tensor> input_scale,
+                                        std::optional<torch::Tensor> weight_scale, std::shared_ptr<ProfilingContext>) {
+  return forward(std::move(input), std::move(weight), std::move(bias), std::move(output), std::move(input_scale),
+                 std::move(weight_scale));
+}
+
 torch::Tensor calc_scatter_index(torch::Tensor choosed_experts, torch::Tensor splits) {
   FLUX_AMD_CHECK_INPUT(choosed_experts, at::kInt);
   FLUX_AMD_CHECK_INPUT(splits, at::kInt);

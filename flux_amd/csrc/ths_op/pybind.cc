@@ -125,7 +125,16 @@ PYBIND11_MODULE(flux_ths_pybind, m) {
            py::arg("output") = py::none(), py::arg("input_scale") = py::none(), py::arg("weight_scale") = py::none())
       .def("forward_grouped", &BlockScaleGemm::forward_grouped, py::arg("input"), py::arg("input_splits"),
            py::arg("weight"), py::arg("bias") = py::none(), py::arg("output") = py::none(),
-           py::arg("input_scale") = py::none(), py::arg("weight_scale") = py::none());
+           py::arg("input_scale") = py::none(), py::arg("weight_scale") = py::none())
+      .def("forward_multistream", &BlockScaleGemm::forward_multistream, py::arg("input"), py::arg("input_splits"),
+           py::arg("weight"), py::arg("bias") = py::none(), py::arg("output") = py::none(),
+           py::arg("input_scale") = py::none(), py::arg("weight_scale") = py::none())
+      .def("reference", &BlockScaleGemm::reference, py::arg("input"), py::arg("weight"), py::arg("bias") = py::none(),
+           py::arg("output") = py::none(), py::arg("input_scale") = py::none(), py::arg("weight_scale") = py::none(),
+           py::arg("is_groupwise_b") = false)
+      .def("profiling", &BlockScaleGemm::profiling, py::arg("input"), py::arg("weight"), py::arg("bias") = py::none(),
+           py::arg("output") = py::none(), py::arg("input_scale") = py::none(), py::arg("weight_scale") = py::none(),
+           py::arg("prof_ctx") = nullptr);
 
   py::class_<Quantization>(m, "Quantization")
       .def(py::init([](py::object input_dtype, py::object output_dtype, int32_t num_streams) {

@@ -107,6 +107,17 @@ class BlockScaleGemm {
   torch::Tensor forward_grouped(torch::Tensor input, torch::Tensor input_splits, torch::Tensor weight,
                                 std::optional<torch::Tensor> bias, std::optional<torch::Tensor> output,
                                 torch::Tensor input_scale, torch::Tensor weight_scale);
+  // The grouped product with input_scale as [M, K/128] (any strides) and weight_scale [E, N/128, K/128]: the
+  // arguments of the reference's multi-stream form; one launch here.
+  torch::Tensor forward_multistream(torch::Tensor input, torch::Tensor input_splits, torch::Tensor weight,
+                                    std::optional<torch::Tensor> bias, std::optional<torch::Tensor> output,
+                                    std::optional<torch::Tensor> input_scale, std::optional<torch::Tensor> weight_scale);
+  torch::Tensor reference(torch::Tensor input, torch::Tensor weight, std::optional<torch::Tensor> bias,
+                          std::optional<torch::Tensor> output, std::optional<torch::Tensor> input_scale,
+                          std::optional<torch::Tensor> weight_scale, bool is_groupwise_b);
+  torch::Tensor profiling(torch::Tensor input, torch::Tensor weight, std::optional<torch::Tensor> bias,
+                          std::optional<torch::Tensor> output, std::optional<torch::Tensor> input_scale,
+                          std::optional<torch::Tensor> weight_scale, std::shared_ptr<ProfilingContext> prof_ctx);
 
  private:
   at::ScalarType input_dtype_, weight_dtype_, output_dtype_;

@@ -324,7 +324,7 @@ def test_sm_margin_through_the_ops(c1):
 
 
 def test_blockscale_gemm_op_dense_and_grouped():
-    """BlockScaleGemm.forward / forward_grouped (src/pybind/gemm_only.cc:77-139) fed by the Quantization op, the way
+    """BlockScaleGemm.forward / forward_grouped / forward_multistream / reference (src/pybind/gemm_only.cc:77-160) fed by the Quantization op, the way
     test/python/gemm_only/test_blockwise_scale_gemm_only.py drives them: both scale layouts of forward_grouped."""
     g = torch.Generator().manual_seed(12)
     experts, n, k = 3, 384, 512
@@ -350,6 +350,17 @@ def test_blockscale_gemm_op_dense_and_grouped():
     d = op.forward(qx, qw[0], input_scale=sx, weight_scale=sw[0].contiguous())
     refd = layers.fp8_blockscale_grouped_gemm_fp32(qx.cpu(), sa, qw.cpu()[:1], sw.cpu()[:1], np.array([m], dtype=np.int32))
     assert torch.allclose(d.float().cpu(), refd, rtol=1e-2, atol=1e-2 * float(refd.abs().max()))
+    # the multi-stream form's arguments (blockscale_gemm.cc:376-486): input_scale [M, K/128] as the transposed view of a
+    # [K/128, M] tensor, weight_scale [E, N/128, K/128]; same launch, same bits
+    sa_t = sa.t().contiguous().cuda().t()
+    assert sa_t.shape == (m, k // 128) and not sa_t.is_contiguous()
+    out3 = op.forward_multistream(qx, torch.from_numpy(split), qw, input_scale=sa_t, weight_scale=sw)
+    assert torch.equal(out3, out)
+    # the reference's second implementation and its tuning entry point: one kernel here
+    assert torch.equal(op.reference(qx, qw[0], input_scale=sx, weight_scale=sw[0].contiguous()), d)
+    assert torch.equal(op.profiling(qx, qw[0], input_scale=sx, weight_scale=sw[0].contiguous()), d)
+    with pytest.raises(RuntimeError, match="is_groupwise_b"):
+        op.reference(qx, qw[0], input_scale=sx, weight_scale=sw[0].contiguous(), is_groupwise_b=True)
     with pytest.raises(RuntimeError, match="bias"):
         op.forward(qx, qw[0], bias=torch.zeros(1, device="cuda"), input_scale=sx, weight_scale=sw[0].contiguous())
     with pytest.raises(RuntimeError, match="cpu"):

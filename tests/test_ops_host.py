@@ -20,7 +20,7 @@ def test_module_exports_reference_names():
                                                     "forward_gather_rs_no_zerobuffer", "ep_zero_buffer", "profiling")),
                          (m.ProfilingContext, ("get_code", "get_all_prof_results", "get_latest_prof_result",
                                                "get_latest_record", "get_all_records")),
-                         (m.BlockScaleGemm, ("forward", "forward_grouped")),
+                         (m.BlockScaleGemm, ("forward", "forward_grouped", "forward_multistream", "reference", "profiling")),
                          (m.Quantization, ("quantize_vector_blockwise", "quantize_square_blockwise",
                                            "batch_quantize_square_blockwise"))):
         for meth in methods:
@@ -43,6 +43,10 @@ def test_keyword_names_match_reference():
         assert kw in doc, kw
     for kw in ("input_dtype", "weight_dtype", "output_dtype", "num_streams"):
         assert kw in m.BlockScaleGemm.__init__.__doc__, kw
+    doc = m.BlockScaleGemm.forward_multistream.__doc__  # src/pybind/gemm_only.cc:110-119
+    for kw in ("input", "input_splits", "weight", "bias", "output", "input_scale", "weight_scale"):
+        assert kw in doc, kw
+    assert "is_groupwise_b" in m.BlockScaleGemm.reference.__doc__ and "prof_ctx" in m.BlockScaleGemm.profiling.__doc__
     doc = m.GemmGroupedV3GatherRS.__init__.__doc__
     for kw in ("total_num_experts", "max_m", "n_dim", "topk", "rank", "world_size", "tp_world_size", "ep_world_size",
                "max_input_groups", "ep_in_dp"):
