@@ -442,6 +442,18 @@ def main():
             adj = PEAK_BF16_TFLOPS * sus["sclk_mhz"] / PEAK_SCLK_MHZ
             roofline["peak_clock_adjusted"] = round(adj, 1)
             roofline["frac_of_clock_adjusted_peak"] = round(sus["tflops"] / adj, 4)
+        # The same two launches on zero-valued operands of the same shapes (same instruction stream, same tile
+        # schedule): without the data's switching activity the board stays under its power limit and the clock is
+        # not lowered, which separates what the kernel's schedule costs from what the power limit costs.  Not a
+        # throughput figure of the workload.
+        xz, w1z, w2z = torch.zeros_like(x), torch.zeros_like(w1), torch.zeros_like(w2)
+        yz, zz = torch.zeros_like(y), torch.empty_like(z)
+        zs = sustained_gemm(torch, lambda: (capi.grouped_gemm(xz, w1z, splits_d, out=yz, gather_a=gather_d),
+                                            capi.grouped_gemm(yz, w2z, splits_d, out=zz, row_scale=row_w)),
+                            min(a.sustain_s, 1.5), step_flops)
+        zs["frac_of_peak"] = round(zs["tflops"] / PEAK_BF16_TFLOPS, 4)
+        roofline["zero_operands_same_launches"] = zs
+        del xz, w1z, w2z, yz, zz
 
     if not a.no_aux:
         kernels.update(aux_measurements(torch, capi, configs, a, wl, dev, gen, (x, w1, w2, y, out, row_w)))
