@@ -31,6 +31,11 @@ HIP_FLAGS = [
     "-Wno-unused-command-line-argument",
 ]
 
+# Per-file additions.  The block-scaled GEMM promotes every MFMA result with vector-ALU instructions right away:
+# its MFMAs must write vector registers (the compiler's default for a kernel that uses both register files is
+# the accumulation registers, which costs a v_accvgpr_read per element and promotion).
+EXTRA_HIP_FLAGS = {"grouped_gemm_fp8_blockscale.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+
 KERNEL_LIB = os.path.join(LIB_DIR, "libfluxmi_kernels.so")
 
 
@@ -78,7 +83,7 @@ def build_kernels(force=True):
         dep = obj[:-2] + ".d"
         if not force and _object_current(obj, dep):
             return obj
-        _run([HIPCC, *HIP_FLAGS, "-MD", "-MF", dep, "-c", os.path.join(KERNEL_DIR, name), "-o", obj])
+        _run([HIPCC, *HIP_FLAGS, *EXTRA_HIP_FLAGS.get(name, []), "-MD", "-MF", dep, "-c", os.path.join(KERNEL_DIR, name), "-o", obj])
         rebuilt.append(name)
         return obj
 

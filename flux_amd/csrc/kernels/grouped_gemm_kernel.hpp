@@ -909,6 +909,276 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
   __builtin_amdgcn_s_barrier();  // the LDS windows are free again before the next tile's fills start
 }
 
+// Block-scaled fp8, one 256 x 128 piece: A carries one scale per row and 128 of K, B one per 128 x 128 block, and
+// the products of every 128 of K are added to the result with a_scale[row] * b_scale (the promotion).
+//
+// The unit of the k loop is a pair of k-steps, i.e. one scale block: LDS rows hold 128 bytes of K, a ring stage is
+// 256 X rows + 128 W rows + the 256 row scales of the pair (49 KiB; three stages).  A wave computes its 128 x 64
+// quarter block by block: for each 32 x 32 block the two MFMAs of the pair (the first with C = 0), then
+// main += block * scale — the block's sums live in vector registers for the length of three MFMAs and the promotion
+// is one v_fmac per element (sums kept in accumulation registers across a whole k-step would cost a register read
+// per element as well: with one wave per SIMD the vector ALU's time adds to the MFMA time).  Fragments of a whole
+// pair are in registers, double-buffered: during pair kb the first half of the MFMA slots issues the fills of pair
+// kb + 2 (stage (kb + 2) % 3), then one wait + barrier makes pair kb + 1 visible (requested during the first half
+// of pair kb - 1), and the second half reads its fragments.  One barrier per 128 of K.
+//
+// A fill instruction covers 8 rows x 128 bytes (whole cache lines); chunk c of row r lies in 16-byte slot
+// c ^ ((r >> 1) & 7) of the row, which makes the 32-row fragment reads free of bank conflicts.
+__device__ __forceinline__ void gemm_tile_blockscaled(const GemmParams &p, uint8_t *smem, const TileCtx &c, const TileDesc &t) {
+  constexpr int XROWS = 256, WROWS = 128, ROWB = 128;
+  constexpr int XBYTES = XROWS * ROWB, WBYTES = WROWS * ROWB;  // 32 KiB, 16 KiB
+  constexpr int SCALE_OFF = XBYTES + WBYTES;                   // 256 floats
+  constexpr int PSB = SCALE_OFF + 1024;                        // bytes of a stage
+  constexpr int NSTG = 3;
+  static_assert(NSTG * PSB <= LDS_BYTES, "three stages fit the LDS");
+  constexpr int XF = 8, WF = 4;          // fill instructions per wave and pair: X rows, W rows
+  constexpr int PAIRF = XF + WF + 1;     // ... with the scale fill
+  constexpr int MBK = 4, NBK = 2, NBLK = MBK * NBK;
+  typedef Geom<1>::Acc Acc;
+  const int wave = c.wave, lane = c.lane, wm = c.wm, wn = c.wn;
+  const int e = t.e, row_base = t.row_base, rows_e = t.rows_e, m0 = t.m0;
+  const int kblocks = c.nk >> 1;
+  const KernArgs pe = kernel_args();
+
+  // ---- operand addressing -------------------------------------------------------------------------------
+  const bool gathered = p.gather_a != nullptr;
+  const uint8_t *xbase = gathered ? p.a : p.a + static_cast<int64_t>(row_base + m0) * c.kbytes;
+  const int64_t xrows = gathered ? p.a_rows : rows_e - m0;
+  const __amdgpu_buffer_rsrc_t xrsrc = make_rsrc(xbase, xrows > 0 ? xrows * c.kbytes : 0xffffffffll);
+  int n0 = t.n0;
+  const int g = split_group(n0, p.n, p.ngroups);
+  const __amdgpu_buffer_rsrc_t wrsrc =
+      make_rsrc(pe->b[g] + (static_cast<int64_t>(e) * p.n + n0) * c.kbytes, static_cast<int64_t>(p.n - n0) * c.kbytes);
+  const __amdgpu_buffer_rsrc_t zrsrc = make_rsrc(g_zero_page, 1024);
+  const uint32_t zoff = (lane & 7) * 16;
+  uint32_t xoff[XF], woff[WF];
+#pragma unroll
+  for (int j = 0; j < XF; ++j) {
+    int xr = m0 + 64 * wave + 8 * j + (lane >> 3);
+    if (xr > rows_e - 1) xr = rows_e - 1;
+    if (xr < 0) xr = 0;
+    int64_t arow = xr - m0;
+    if (gathered) {
+      arow = p.gather_a[row_base + xr];
+      if (p.a_rows > 0) arow = arow < 0 ? 0 : (arow >= p.a_rows ? p.a_rows - 1 : arow);
+    }
+    const int chunk = (lane & 7) ^ ((4 * j + (lane >> 4)) & 7);
+    xoff[j] = static_cast<uint32_t>(arow * c.kbytes) + chunk * 16;
+  }
+#pragma unroll
+  for (int j = 0; j < WF; ++j) {
+    int wr = n0 + 32 * wave + 8 * j + (lane >> 3);
+    if (wr > p.n - 1) wr = p.n - 1;
+    const int chunk = (lane & 7) ^ ((4 * j + (lane >> 4)) & 7);
+    woff[j] = static_cast<uint32_t>((wr - n0) * c.kbytes) + chunk * 16;
+  }
+  // Scales: lane l of a wave fetches the scale of tile row 64 * wave + l.
+  const __amdgpu_buffer_rsrc_t as_rsrc = make_rsrc(reinterpret_cast<const uint8_t *>(pe->a_scale), 0xffffffffll);
+  uint32_t as_voff;
+  int as_kstep, bs_base, bs_kstep;
+  {
+    int xr = m0 + 64 * wave + lane;
+    if (xr > rows_e - 1) xr = rows_e - 1;
+    int64_t arow = row_base + xr;
+    if (gathered) {
+      arow = p.gather_a[row_base + xr];
+      if (p.a_rows > 0) arow = arow < 0 ? 0 : (arow >= p.a_rows ? p.a_rows - 1 : arow);
+    }
+    if (pe->a_scale_layout == FLUXMI_ASCALE_BLOCK128) {  // [ceil(rows/128), K/128, 128], row in block fastest
+      as_voff = static_cast<uint32_t>(((arow >> 7) * kblocks * 128 + (arow & 127)) * 4);
+      as_kstep = 128 * 4;
+    } else {  // per expert [K/128, rows of the expert], experts back to back
+      as_voff = static_cast<uint32_t>((static_cast<int64_t>(row_base) * kblocks + xr) * 4);
+      as_kstep = rows_e * 4;
+    }
+    const int nb = n0 >> 7, nblocks = (pe->n + 127) >> 7;
+    if (pe->b_scale_layout == FLUXMI_BSCALE_N_K) {  // [E, N/128, K/128]
+      bs_base = (e * nblocks + nb) * kblocks;
+      bs_kstep = 1;
+    } else {  // [E, K/128, N/128]
+      bs_base = e * kblocks * nblocks + nb;
+      bs_kstep = nblocks;
+    }
+  }
+  typedef const __attribute__((address_space(4))) float *ConstF32;
+  const ConstF32 bscale = (ConstF32)(pe->b_scale);
+  auto bscale_of = [&](int kb) { return bscale[__builtin_amdgcn_readfirstlane(bs_base + (kb < kblocks ? kb : 0) * bs_kstep)]; };
+
+  // Fill instruction Q of pair kb into stage STAGE: the scale fill first, then X row groups, then W row groups.
+  // Past the end of K the fills read the zero page (the fill counts of the waits must hold).
+  uint8_t *const xdst = smem + (XF * wave) * 1024;
+  uint8_t *const wdst = smem + XBYTES + (WF * wave) * 1024;
+  auto fill = [&](auto STAGE, auto Q, int kb) {
+    constexpr int stage = decltype(STAGE)::value, q = decltype(Q)::value;
+    const bool in = kb < kblocks;
+    if constexpr (q == 0)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(in ? as_rsrc : zrsrc, (lds_ptr_t)(smem + stage * PSB + SCALE_OFF + wave * 256), 4,
+                                               static_cast<int>(in ? as_voff : static_cast<uint32_t>(lane * 4)),
+                                               in ? kb * as_kstep : 0, 0, 0);
+    else if constexpr (q <= XF)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(in ? xrsrc : zrsrc, (lds_ptr_t)(xdst + stage * PSB + (q - 1) * 1024), 16,
+                                               static_cast<int>(in ? xoff[q - 1] : zoff), in ? kb * ROWB : 0, 0, 0);
+    else
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(in ? wrsrc : zrsrc, (lds_ptr_t)(wdst + stage * PSB + (q - 1 - XF) * 1024), 16,
+                                               static_cast<int>(in ? woff[q - 1 - XF] : zoff), in ? kb * ROWB : 0, 0, 0);
+  };
+
+  // Fragments of a pair: block b of an operand, k-step h of the pair, 16-byte chunk s (a 32x32x64 MFMA takes two).
+  // Lane l reads row l & 31 of the block, logical chunk 4 h + 2 (l >> 5) + s.
+  struct Frags {
+    i32x4 x[MBK][2][2], w[NBK][2][2];
+  };
+  Frags fa, fb;
+  float sa[MBK], sb[MBK];  // row scales of the pair, as read
+  uint32_t roff[2][2];     // byte offset of (h, s) inside a 32-row block, this lane
+#pragma unroll
+  for (int h = 0; h < 2; ++h)
+#pragma unroll
+    for (int s2 = 0; s2 < 2; ++s2) {
+      const int r = lane & 31, ch = 4 * h + 2 * (lane >> 5) + s2;
+      roff[h][s2] = r * ROWB + ((ch ^ ((r >> 1) & 7)) << 4);
+    }
+  const uint8_t *const xread = smem + wm * 128 * ROWB;
+  const uint8_t *const wread = smem + XBYTES + wn * 64 * ROWB;
+  const float *const sread = reinterpret_cast<const float *>(smem + SCALE_OFF) + wm * 128 + (lane & 31);
+  // Read number R (0 .. 25) of the pair in stage STAGE: 16 X chunks, 8 W chunks, then the row scales (2 x 2).
+  auto read_one = [&](auto STAGE, auto R, Frags &f, float (&sc)[MBK]) {
+    constexpr int stage = decltype(STAGE)::value, r = decltype(R)::value;
+    if constexpr (r < 16) {
+      constexpr int i = r >> 2, h = (r >> 1) & 1, s2 = r & 1;
+      f.x[i][h][s2] = *reinterpret_cast<const i32x4 *>(xread + stage * PSB + i * 32 * ROWB + roff[h][s2]);
+    } else if constexpr (r < 24) {
+      constexpr int j = (r - 16) >> 2, h = ((r - 16) >> 1) & 1, s2 = (r - 16) & 1;
+      f.w[j][h][s2] = *reinterpret_cast<const i32x4 *>(wread + stage * PSB + j * 32 * ROWB + roff[h][s2]);
+    } else {
+      constexpr int i0 = (r - 24) * 2;
+      sc[i0] = sread[stage * (PSB / 4) + i0 * 32];
+      sc[i0 + 1] = sread[stage * (PSB / 4) + (i0 + 1) * 32];
+    }
+  };
+  constexpr int NREADS = 26;
+
+  Acc main_acc[MBK][NBK];
+#pragma unroll
+  for (int i = 0; i < MBK; ++i)
+#pragma unroll
+    for (int j = 0; j < NBK; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) main_acc[i][j][v] = 0.f;
+
+  auto mfma = [&](const Frags &f, int i, int j, int h, Acc cacc) {
+    i32x8 wa, xa;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      wa[v] = f.w[j][h][0][v];
+      wa[4 + v] = f.w[j][h][1][v];
+      xa[v] = f.x[i][h][0][v];
+      xa[4 + v] = f.x[i][h][1][v];
+    }
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wa, xa, cacc, 0, 0, 0, 0, 0, 0);
+  };
+
+  // One pair of k-steps, number U within a run of six (three stages x two fragment sets): MFMAs on `cur`, the
+  // fragments and scales of the next pair into `nxt`.  MFMA slot t: blocks two at a time, (b, k0) (b+1, k0) (b, k1)
+  // (b+1, k1), so that the second MFMA of a block does not follow its first directly; block b is promoted two slots
+  // after its second MFMA.
+  float bsv_next = 0.f;
+  auto pair_step = [&](auto U, int kb0, const Frags &cur, const float (&scur)[MBK], Frags &nxt, float (&snxt)[MBK], float bsv) {
+    constexpr int u = decltype(U)::value;
+    const int kb = kb0 + u;
+    float psc[MBK];
+#pragma unroll
+    for (int i = 0; i < MBK; ++i) psc[i] = scur[i] * bsv;
+    bsv_next = bscale_of(kb + 1);
+    Acc blk[NBLK];
+    static_for<0, 2 * NBLK>([&](auto T) {
+      constexpr int tt = decltype(T)::value;
+      constexpr int b = (tt >> 2) * 2 + (tt & 1), h = (tt >> 1) & 1;
+      if constexpr (tt < NBLK) {
+        // first half: the fills of pair kb + 2
+        static_for<0, PAIRF>([&](auto Q) {
+          constexpr int q = decltype(Q)::value;
+          if constexpr (q * NBLK / PAIRF == tt) fill(std::integral_constant<int, (u + 2) % NSTG>{}, Q, kb + 2);
+        });
+      } else {
+        if constexpr (tt == NBLK) {
+          // pair kb + 1 has landed (everything but the fills just issued), for every wave's share
+          FLUXMI_WAITCNT(PAIRF, 15);
+          __builtin_amdgcn_s_barrier();
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        static_for<0, NREADS>([&](auto R) {
+          constexpr int r = decltype(R)::value;
+          if constexpr (r * NBLK / NREADS == tt - NBLK) read_one(std::integral_constant<int, (u + 1) % NSTG>{}, R, nxt, snxt);
+        });
+      }
+      if constexpr (h == 0) blk[b] = mfma(cur, b / NBK, b % NBK, 0, Acc{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f});
+      else blk[b] = mfma(cur, b / NBK, b % NBK, 1, blk[b]);
+      // promotion of the block whose second MFMA was issued two slots ago
+      if constexpr (tt >= 4 && ((tt - 2) >> 1 & 1) == 1) {
+        constexpr int pb = ((tt - 2) >> 2) * 2 + ((tt - 2) & 1);
+#pragma unroll
+        for (int v = 0; v < 16; ++v) main_acc[pb / NBK][pb % NBK][v] = fmaf(blk[pb][v], psc[pb / NBK], main_acc[pb / NBK][pb % NBK][v]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    // the last two blocks
+    static_for<NBLK - 2, NBLK>([&](auto B) {
+      constexpr int pb = decltype(B)::value;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) main_acc[pb / NBK][pb % NBK][v] = fmaf(blk[pb][v], psc[pb / NBK], main_acc[pb / NBK][pb % NBK][v]);
+    });
+    FLUXMI_WAITCNT(63, 0);  // the fragments of the next pair are in registers
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  // ---- prologue: pairs 0 and 1 requested, pair 0 read ---------------------------------------------------
+  FLUXMI_WAITCNT(0, 0);  // stores of the previous tile's epilogue
+  static_for<0, PAIRF>([&](auto Q) { fill(std::integral_constant<int, 0>{}, Q, 0); });
+  static_for<0, PAIRF>([&](auto Q) { fill(std::integral_constant<int, 1>{}, Q, 1); });
+  float bsv = bscale_of(0);
+  FLUXMI_WAITCNT(PAIRF, 15);
+  __builtin_amdgcn_s_barrier();
+  static_for<0, NREADS>([&](auto R) { read_one(std::integral_constant<int, 0>{}, R, fa, sa); });
+  FLUXMI_WAITCNT(63, 0);
+
+  // ---- main loop: six pairs per trip, pairs past the end of K skipped ------------------------------------
+  // (A skipped pair issues no fills either: the waits count the fills of executed pairs only, and those are the
+  // same for every wave.)
+  for (int kb0 = 0; kb0 < kblocks; kb0 += 6) {
+    pair_step(std::integral_constant<int, 0>{}, kb0, fa, sa, fb, sb, bsv);
+    bsv = bsv_next;
+    if (kb0 + 1 < kblocks) { pair_step(std::integral_constant<int, 1>{}, kb0, fb, sb, fa, sa, bsv); bsv = bsv_next; }
+    if (kb0 + 2 < kblocks) { pair_step(std::integral_constant<int, 2>{}, kb0, fa, sa, fb, sb, bsv); bsv = bsv_next; }
+    if (kb0 + 3 < kblocks) { pair_step(std::integral_constant<int, 3>{}, kb0, fb, sb, fa, sa, bsv); bsv = bsv_next; }
+    if (kb0 + 4 < kblocks) { pair_step(std::integral_constant<int, 4>{}, kb0, fa, sa, fb, sb, bsv); bsv = bsv_next; }
+    if (kb0 + 5 < kblocks) { pair_step(std::integral_constant<int, 5>{}, kb0, fb, sb, fa, sa, bsv); bsv = bsv_next; }
+  }
+
+  // ---- epilogue -------------------------------------------------------------------------------------------
+  FLUXMI_WAITCNT(0, 0);          // this wave's trailing fills have landed
+  __builtin_amdgcn_s_barrier();  // ... and everybody else's; nobody reads the ring any more
+  uint8_t *windows = smem + wave * 8192;  // one 8 KiB window per wave
+  const int wrow0 = m0 + wm * 128;
+  {
+    const int wcol0 = n0 + wn * 64;
+    const bool full = wrow0 + 128 <= rows_e && wcol0 + 64 <= pe->n && pe->scatter_d == nullptr && pe->accumulate == 0;
+    const bool out_f32 = pe->d_fp32 != 0;
+    const bool scaled = !(c.scalar == 1.f && pe->alpha[g] == nullptr && pe->row_scale == nullptr && pe->col_scale == nullptr);
+    if (full && !scaled) {
+      if (out_f32) store_tile<1, 4, 2, true, true, false>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, main_acc);
+      else store_tile<1, 4, 2, true, false, false>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, main_acc);
+    } else if (full) {
+      if (out_f32) store_tile<1, 4, 2, true, true, true>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, main_acc);
+      else store_tile<1, 4, 2, true, false, true>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, main_acc);
+    } else {
+      if (out_f32) store_tile<1, 4, 2, false, true, true>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, main_acc);
+      else store_tile<1, 4, 2, false, false, true>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, main_acc);
+    }
+  }
+  __builtin_amdgcn_s_barrier();  // the LDS windows are free again before the next tile's fills start
+}
+
 template <int ELT, bool BS = false>
 __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmParams p) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];  // STAGES x (X tile | W tile)
@@ -1065,7 +1335,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
     item += grid;
     const TileDesc next = locate(item);
     if constexpr (BS) {
-      if (cur.kind == 2) gemm_tile<ELT, 4, 2, true>(p, smem, c, cur, next, pf);
+      if (cur.kind == 2) gemm_tile_blockscaled(p, smem, c, cur);
     } else {
       if (cur.kind == 0) gemm_tile<ELT, 4, 4>(p, smem, c, cur, next, pf);
       else if (cur.kind == 1) gemm_tile<ELT, 2, 4>(p, smem, c, cur, next, pf);
