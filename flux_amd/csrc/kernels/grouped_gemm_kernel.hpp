@@ -107,6 +107,12 @@ __device__ __forceinline__ float acc_read(float a) {
   return v;
 }
 
+template <bool IN_VGPR>
+__device__ __forceinline__ float sum_read(float a) {
+  if constexpr (IN_VGPR) return a;
+  else return acc_read(a);
+}
+
 // Compile-time loop: f(integral_constant<int, I>) for I in [0, N).
 template <int I, int N, class F>
 __device__ __forceinline__ void static_for(F &&f) {
@@ -122,7 +128,9 @@ __device__ __forceinline__ void static_for(F &&f) {
 // row (j below counts 32-column groups, ip 64-row groups).  FULL: every row and column of the wave's quarter exists and rows are stored where they are (no
 // scatter), so no store is predicated.  OUT_F32 selects the output element type.  !SCALED: every scale
 // factor is 1 and the multiplications are left out.
-template <int ELT, int MB, int NB, bool FULL, bool OUT_F32, bool SCALED>
+// SUMS_IN_VGPRS: the sums are ordinary vector-register values (the block-scaled kernel's promoted sums) and are
+// read as they are.
+template <int ELT, int MB, int NB, bool FULL, bool OUT_F32, bool SCALED, bool SUMS_IN_VGPRS = false>
 __device__ __forceinline__ void store_tile(uint8_t *windows, const TileCtx &c, int g, int e, int row_base, int rows_e,
                                            int wrow0, int wcol0,
                                            const typename Geom<ELT>::Acc (&acc)[32 * MB / Geom<ELT>::BLK][32 * NB / Geom<ELT>::BLK]) {
@@ -178,8 +186,8 @@ __device__ __forceinline__ void store_tile(uint8_t *windows, const TileCtx &c, i
             for (int ii = 0; ii < 4; ++ii) {
               const int i = ip * 4 + ii;
               const int r = ii * 16 + (lane & 15);
-              float4 v = make_float4(acc_read(acc[i][jb][0]), acc_read(acc[i][jb][1]), acc_read(acc[i][jb][2]),
-                                     acc_read(acc[i][jb][3]));
+              float4 v = make_float4(sum_read<SUMS_IN_VGPRS>(acc[i][jb][0]), sum_read<SUMS_IN_VGPRS>(acc[i][jb][1]), sum_read<SUMS_IN_VGPRS>(acc[i][jb][2]),
+                                     sum_read<SUMS_IN_VGPRS>(acc[i][jb][3]));
               if constexpr (SCALED) {
                 v = make_float4(v.x * rs[i], v.y * rs[i], v.z * rs[i], v.w * rs[i]);
                 v = make_float4(v.x * cs.x, v.y * cs.y, v.z * cs.z, v.w * cs.w);
@@ -232,8 +240,8 @@ __device__ __forceinline__ void store_tile(uint8_t *windows, const TileCtx &c, i
 #pragma unroll
         for (int q = 0; q < Geom<ELT>::NACC / 4; ++q) {
           const int chunk = BLK == 32 ? 2 * q + h : jj * 4 + (lane >> 4);
-          float4 v = make_float4(acc_read(acc[i][jb][4 * q + 0]), acc_read(acc[i][jb][4 * q + 1]),
-                                 acc_read(acc[i][jb][4 * q + 2]), acc_read(acc[i][jb][4 * q + 3]));
+          float4 v = make_float4(sum_read<SUMS_IN_VGPRS>(acc[i][jb][4 * q + 0]), sum_read<SUMS_IN_VGPRS>(acc[i][jb][4 * q + 1]),
+                                 sum_read<SUMS_IN_VGPRS>(acc[i][jb][4 * q + 2]), sum_read<SUMS_IN_VGPRS>(acc[i][jb][4 * q + 3]));
           if constexpr (SCALED) v = make_float4(v.x * rs[i], v.y * rs[i], v.z * rs[i], v.w * rs[i]);
           *reinterpret_cast<float4 *>(half + r * 128 + ((chunk ^ ((r >> 1) & 7)) << 4)) = v;
         }
@@ -483,16 +491,9 @@ __device__ __forceinline__ void issue_first_pairs(const TileOperands<XL, WL> &op
 // (MB, NB) = (4, 4) is the macro tile, (2, 4) its upper half (for the last rows of an expert); (4, 2) and
 // (2, 2) are the 256x128 and 128x128 pieces a tile of the last, partly filled round is cut into.  Waves
 // are laid out 2 x 2.
-//
-// BS (block-scaled fp8, 256 x 128 tiles only): A carries one scale per row and 128 of K, B one per 128 x 128
-// block.  A pair of k-steps is one scale block of K: its products are summed in `acc`, and at the end of the
-// pair main += acc * a_scale[row] * b_scale, acc = 0.  The 256 row scales of a pair travel like its operands: one
-// more direct-to-LDS fill per wave (64 rows x 4 bytes), the first instruction of the pair's fills, into the
-// half of the pair's first ring stage that a 128-column W tile leaves unused; the wait counts below include it.
-template <int ELT, int MB, int NB, bool BS = false>
+template <int ELT, int MB, int NB>
 __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, const TileCtx &c, const TileDesc &t,
                                           const TileDesc &next, TilePrefetch &pf) {
-  static_assert(!BS || (ELT == 1 && MB == 4 && NB == 2), "block scales: fp8, 256 x 128 tiles");
   constexpr int XLOADS = MB;           // direct-to-LDS instructions per wave per stage, X tile
   constexpr int WLOADS = NB;           // same, W tile
   constexpr int LOADS = XLOADS + WLOADS;
@@ -502,11 +503,10 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
   constexpr int NR = (MBK + NBK) * NCH;  // fragment reads per k-step (16 bytes per lane each)
   constexpr int NM = MBK * NBK;          // MFMAs per k-step
   constexpr int RSPAN = NM / 2;        // MFMA slots over which the fragment reads of a step are spread
-  constexpr int PAIR = 2 * LOADS + (BS ? 1 : 0);  // vector-memory instructions per wave and pair of k-steps
-  constexpr int HALF = LOADS + (BS ? 1 : 0);      // ... of which the pair's first step issues this many
+  constexpr int PAIR = 2 * LOADS;  // vector-memory instructions per wave and pair of k-steps
+  constexpr int HALF = LOADS;      // ... of which the pair's first step issues this many
   constexpr int WAIT_EVEN = (LA - 2) / 2 * PAIR;  // outstanding fills allowed when an even step starts
   constexpr int WAIT_ODD = (LA - 4) / 2 * PAIR + HALF;
-  constexpr int SCALE_OFF = XB + W_TILE_BYTES / 2;  // row scales of a pair inside its first stage (BS)
   const int wave = c.wave, lane = c.lane, wm = c.wm, wn = c.wn, nk = c.nk;
   const int e = t.e, row_base = t.row_base, rows_e = t.rows_e, m0 = t.m0;
 
@@ -605,90 +605,6 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
 #pragma unroll
       for (int v = 0; v < Geom<ELT>::NACC; ++v) acc[i][j][v] = 0.f;
 
-  // ---- block scales (BS only) ------------------------------------------------------------------------
-  // main: the promoted sums.  Lane l of the scale fill fetches the scale of tile row 64 * wave + l; a scale block
-  // kb of K adds as_kstep bytes to every lane's offset.  b_scale: one value per pair, a scalar load.
-  typename Geom<ELT>::Acc main_acc[BS ? MBK : 1][BS ? NBK : 1];
-  __amdgpu_buffer_rsrc_t as_rsrc = zrsrc;
-  uint32_t as_voff = 0;
-  int as_kstep = 0, bs_base = 0, bs_kstep = 0;
-  const int kblocks = nk >> 1;
-  if constexpr (BS) {
-#pragma unroll
-    for (int i = 0; i < MBK; ++i)
-#pragma unroll
-      for (int j = 0; j < NBK; ++j)
-#pragma unroll
-        for (int v = 0; v < Geom<ELT>::NACC; ++v) main_acc[i][j][v] = 0.f;
-    const KernArgs pe = kernel_args();
-    as_rsrc = make_rsrc(reinterpret_cast<const uint8_t *>(pe->a_scale), 0xffffffffll);
-    int xr = m0 + 64 * wave + lane;
-    if (xr > rows_e - 1) xr = rows_e - 1;
-    int64_t arow = row_base + xr;
-    if (pe->gather_a != nullptr) {
-      arow = pe->gather_a[row_base + xr];
-      if (pe->a_rows > 0) arow = arow < 0 ? 0 : (arow >= pe->a_rows ? pe->a_rows - 1 : arow);
-    }
-    if (pe->a_scale_layout == FLUXMI_ASCALE_BLOCK128) {  // [ceil(rows/128), K/128, 128], row in block fastest
-      as_voff = static_cast<uint32_t>(((arow >> 7) * kblocks * 128 + (arow & 127)) * 4);
-      as_kstep = 128 * 4;
-    } else {  // per expert [K/128, rows of the expert], experts back to back
-      as_voff = static_cast<uint32_t>((static_cast<int64_t>(row_base) * kblocks + xr) * 4);
-      as_kstep = rows_e * 4;
-    }
-    int n0g = t.n0;
-    split_group(n0g, pe->n, pe->ngroups);
-    const int nb = n0g >> 7, nblocks = (pe->n + 127) >> 7;
-    if (pe->b_scale_layout == FLUXMI_BSCALE_N_K) {  // [E, N/128, K/128]
-      bs_base = (e * nblocks + nb) * kblocks;
-      bs_kstep = 1;
-    } else {  // [E, K/128, N/128]
-      bs_base = e * kblocks * nblocks + nb;
-      bs_kstep = nblocks;
-    }
-  }
-  // The scale fill of scale block kb into ring slot `slot` (one instruction per wave, also past the end of K,
-  // where it reads zeros: the fill counts of the waits must hold).
-  auto scale_fill = [&](int slot, int kb) {
-    const bool in = kb < kblocks;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(in ? as_rsrc : zrsrc, (lds_ptr_t)(smem + slot * SB + SCALE_OFF + wave * 256), 4,
-                                             static_cast<int>(in ? as_voff : static_cast<uint32_t>(lane * 4)),
-                                             in ? kb * as_kstep : 0, 0, 0);
-  };
-  // The block scale of B for scale block kb: one value per pair of k-steps, fetched with a scalar load when the
-  // pair starts (through the constant address space: as a vector load it would sit in the queue of the ring fills,
-  // and waiting for it would drain them all) and used when the pair ends.
-  typedef const __attribute__((address_space(4))) float *ConstF32;
-  float bsv = 0.f;
-  auto bscale_load = [&](int kb) {
-    if constexpr (BS) {
-      const ConstF32 bs = (ConstF32)(kernel_args()->b_scale);
-      bsv = bs[__builtin_amdgcn_readfirstlane(bs_base + (kb < kblocks ? kb : 0) * bs_kstep)];
-    }
-  };
-  // Promotion of a pair of k-steps: main += acc * (row scale * block scale of B), acc = 0, block by block during the
-  // pair's second step: block b is promoted two MFMA slots after its last MFMA was issued, in the shadow of the
-  // MFMAs of the blocks after it; the last two blocks follow the step.
-  constexpr int PROMOTE_LAG = 2;
-  float psc[BS ? MBK : 1];
-  auto promote_begin = [&](int slot) {
-    if constexpr (BS) {
-      const float *srow = reinterpret_cast<const float *>(smem + slot * SB + SCALE_OFF) + wm * (32 * MB) + (lane & 31);
-#pragma unroll
-      for (int i = 0; i < MBK; ++i) psc[i] = srow[i * 32] * bsv;
-    }
-  };
-  auto promote_block = [&](auto B) {
-    if constexpr (BS) {
-      constexpr int b = decltype(B)::value, i = b / NBK, j = b % NBK;
-#pragma unroll
-      for (int v = 0; v < Geom<ELT>::NACC; ++v) {
-        main_acc[i][j][v] = fmaf(acc[i][j][v], psc[i], main_acc[i][j][v]);
-        acc[i][j][v] = 0.f;
-      }
-    }
-  };
-
   // Fragment addresses: per lane and 16-byte chunk s a base for each operand; a stage and block add a
   // compile-time offset.  LDS instructions carry 16 bits of offset, so three bases 64 KiB apart.
   const uint8_t *xfrag[3][NCH], *wfrag[3][NCH];
@@ -735,10 +651,6 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
     }
     __builtin_amdgcn_s_barrier();     // ... for every wave's share; and everybody is done reading stage u
     __builtin_amdgcn_sched_barrier(0);
-    if constexpr (BS && even) {
-      scale_fill((e0 + LA) % STG, (kbase / KBYTES + e0 + LA) >> 1);
-      bscale_load((kbase / KBYTES + e0) >> 1);
-    }
     static_for<0, NM>([&](auto T) {
       constexpr int t = decltype(T)::value;
       static_for<0, NR>([&](auto R) {
@@ -764,14 +676,9 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
         if constexpr (at % NM != 0 && at - 1 == t + (even ? 0 : NM))
           fill_m0(std::integral_constant<int, (e0 + LA + (d & 1)) % STG>{}, std::integral_constant<int, (d >> 1)>{});
       });
-      if constexpr (BS && !even && t == 0) promote_begin(e0 % STG);
       mfma_slot<ELT, MBK, NBK>(t, xc, wc, acc);
-      if constexpr (BS && !even && t >= PROMOTE_LAG) promote_block(std::integral_constant<int, (t >= PROMOTE_LAG ? t - PROMOTE_LAG : 0)>{});
       __builtin_amdgcn_sched_barrier(0);
     });
-    if constexpr (BS && !even) {
-      static_for<NM - PROMOTE_LAG, NM>([&](auto B) { promote_block(B); });
-    }
     FLUXMI_WAITCNT(63, 0);  // the fragments of the next step are in registers (requested long ago)
     __builtin_amdgcn_sched_barrier(0);
   };
@@ -787,12 +694,6 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
     __builtin_amdgcn_sched_barrier(0);
     const int e0 = even ? ks : ks - 1;
     const int rslot = (ks + 1) % STG, pslot0 = (e0 + LA) % STG, pslot1 = (e0 + LA + 1) % STG;
-    if constexpr (BS) {
-      if (even) {
-        scale_fill(pslot0, (e0 + LA) >> 1);
-        bscale_load(e0 >> 1);
-      }
-    }
     static_for<0, NM>([&](auto T) {
       constexpr int t = decltype(T)::value;
       static_for<0, NR>([&](auto R) {
@@ -808,38 +709,16 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
           if (at - NM == t && !even) fill_dyn((d & 1) ? pslot1 : pslot0, std::integral_constant<int, (d >> 1)>{}, e0 + LA + (d & 1));
         }
       });
-      if constexpr (BS && t == 0) {
-        if (!even) promote_begin(e0 % STG);
-      }
       mfma_slot<ELT, MBK, NBK>(t, xc, wc, acc);
-      if constexpr (BS && t >= PROMOTE_LAG) {
-        if (!even) promote_block(std::integral_constant<int, (t >= PROMOTE_LAG ? t - PROMOTE_LAG : 0)>{});
-      }
       __builtin_amdgcn_sched_barrier(0);
     });
-    if constexpr (BS) {
-      if (!even) static_for<NM - PROMOTE_LAG, NM>([&](auto B) { promote_block(B); });
-    }
     FLUXMI_WAITCNT(63, 0);
     __builtin_amdgcn_sched_barrier(0);
   };
 
   // ---- prologue: k-steps 0..3 requested as two pairs, here or by the previous tile ahead of its epilogue --
   FLUXMI_WAITCNT(0, 0);  // stores of the previous tile's epilogue (and, if it requested them, the first fills)
-  if constexpr (BS) {
-    // Pair by pair like issue_first_pairs, each pair led by its scale fill.
-#pragma unroll
-    for (int s0 = 0; s0 < LA; s0 += 2) {
-      scale_fill(s0, s0 >> 1);
-#pragma unroll
-      for (int q = 0; q < LOADS; ++q) {
-        fill_any<XLOADS, WLOADS>(op, smem, c, q, s0, s0);
-        fill_any<XLOADS, WLOADS>(op, smem, c, q, s0 + 1, s0 + 1);
-      }
-    }
-  } else {
-    if (!prefetched) issue_first_pairs<XLOADS, WLOADS>(op, smem, c);
-  }
+  if (!prefetched) issue_first_pairs<XLOADS, WLOADS>(op, smem, c);
   FLUXMI_WAITCNT(WAIT_EVEN, 15);
   __builtin_amdgcn_s_barrier();
   static_for<0, NR>([&](auto R) { read_one(std::integral_constant<int, 0>{}, R, xa, wa); });
@@ -903,8 +782,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
         else store_tile<ELT, MB, NB, false, false, true>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, res);
       }
     };
-    if constexpr (BS) store(main_acc);
-    else store(acc);
+    store(acc);
   }
   __builtin_amdgcn_s_barrier();  // the LDS windows are free again before the next tile's fills start
 }
@@ -1166,14 +1044,14 @@ __device__ __forceinline__ void gemm_tile_blockscaled(const GemmParams &p, uint8
     const bool out_f32 = pe->d_fp32 != 0;
     const bool scaled = !(c.scalar == 1.f && pe->alpha[g] == nullptr && pe->row_scale == nullptr && pe->col_scale == nullptr);
     if (full && !scaled) {
-      if (out_f32) store_tile<1, 4, 2, true, true, false>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, main_acc);
-      else store_tile<1, 4, 2, true, false, false>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, main_acc);
+      if (out_f32) store_tile<1, 4, 2, true, true, false, true>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, main_acc);
+      else store_tile<1, 4, 2, true, false, false, true>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, main_acc);
     } else if (full) {
-      if (out_f32) store_tile<1, 4, 2, true, true, true>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, main_acc);
-      else store_tile<1, 4, 2, true, false, true>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, main_acc);
+      if (out_f32) store_tile<1, 4, 2, true, true, true, true>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, main_acc);
+      else store_tile<1, 4, 2, true, false, true, true>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, main_acc);
     } else {
-      if (out_f32) store_tile<1, 4, 2, false, true, true>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, main_acc);
-      else store_tile<1, 4, 2, false, false, true>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, main_acc);
+      if (out_f32) store_tile<1, 4, 2, false, true, true, true>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, main_acc);
+      else store_tile<1, 4, 2, false, false, true, true>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, main_acc);
     }
   }
   __builtin_amdgcn_s_barrier();  // the LDS windows are free again before the next tile's fills start
