@@ -32,7 +32,9 @@ def make_case(seed, experts, rows, n, k, empty=()):
 @pytest.mark.parametrize("experts,rows,n,k,seed,empty", [
     (1, 256, 128, 128, 0, ()), (1, 300, 264, 256, 1, ()), (4, 1000, 512, 384, 2, ()), (8, 2048, 1024, 1024, 3, (0, 5)),
     (3, 700, 1408, 2048, 4, (1,)), (16, 900, 256, 640, 5, (2, 3, 15)), (2, 17, 8, 128, 6, ()), (5, 1, 520, 1280, 7, (0, 1, 2, 4)),
-    (2, 600, 640, 1792, 8, ()), (3, 5000, 4096, 512, 9, ()), (1, 130, 136, 2816, 10, ())])
+    (2, 600, 640, 1792, 8, ()), (3, 5000, 4096, 512, 9, ()), (1, 130, 136, 2816, 10, ()),
+    # six and seven scale blocks of K: the last pair of an unrolled trip of the k loop and the first of the next
+    (2, 515, 384, 768, 11, ()), (3, 777, 392, 896, 12, (1,))])
 def test_blockscale_against_oracle_both_layouts(experts, rows, n, k, seed, empty):
     from flux_amd import capi
     print(f"[case] blockscale E={experts} rows={rows} N={n} K={k} empty={empty}", flush=True)
