@@ -47,8 +47,9 @@ def parse():
     ap.add_argument("--no-aux", action="store_true", help="skip the measurements outside the step")
     ap.add_argument("--sustain-s", type=float, default=2.5,
                     help="seconds of the sustained GEMM loop during which the shader clock is sampled (0 = skip)")
-    ap.add_argument("--calib-copy", action="store_true",
-                    help="also run a plain 1 GiB device copy (known traffic) to calibrate rocprofv3 byte counters")
+    ap.add_argument("--no-calib", action="store_true",
+                    help="skip the plain streaming kernels of known traffic (what this box gives a copy / a read "
+                         "stream; also the calibration of the rocprofv3 byte counters)")
     return ap.parse_args()
 
 
@@ -179,9 +180,10 @@ def sustained_gemm(torch, fn, seconds, flops_per_call):
     return out
 
 
-def cpu_baseline(torch, wl_name, x, w1, w2):
+def cpu_baseline(torch, wl_name, x, w1, w2, passes=3):
     """The CPU oracle (PyTorch-CPU restatement of the reference's torch layer) on a bounded sample:
-    one pass over the first `sample_tokens` tokens of the same workload (all of C3), full hidden / ffn sizes."""
+    one warm-up pass and `passes` timed passes over the first `sample_tokens` tokens of the same workload (all of
+    C3), full hidden / ffn sizes; the median pass is reported."""
     from oracle import configs, layers
 
     sample_tokens = {"C1": 256, "C3": 8192, "C4": 8192}[wl_name]
@@ -189,16 +191,24 @@ def cpu_baseline(torch, wl_name, x, w1, w2):
     threads = torch.get_num_threads()
     xs = x[:sample_tokens].cpu()
     w1c, w2c = w1.cpu(), w2.cpu()
-    t0 = time.perf_counter()
-    y = layers.layer0_fp32(xs, w1c, wl.splits, wl.gather_index).to(torch.bfloat16)
-    out = layers.layer1_fp32(y, w2c, wl.splits, wl.scatter_index.reshape(-1), wl.topk,
-                             output_vec_scale=wl.row_weight)
-    dt = time.perf_counter() - t0
+
+    def one_pass():
+        t0 = time.perf_counter()
+        y = layers.layer0_fp32(xs, w1c, wl.splits, wl.gather_index).to(torch.bfloat16)
+        out = layers.layer1_fp32(y, w2c, wl.splits, wl.scatter_index.reshape(-1), wl.topk,
+                                 output_vec_scale=wl.row_weight)
+        dt = time.perf_counter() - t0
+        assert out.shape == (sample_tokens, wl.hidden)
+        return dt
+
+    one_pass()                                   # warm-up: thread pool, page faults of the temporaries
+    times = [one_pass() for _ in range(passes)]  # timed passes
+    dt = statistics.median(times)
     flops = 2.0 * wl.rows * wl.hidden * wl.ffn * 2
-    assert out.shape == (sample_tokens, wl.hidden)
     return {"value": round(flops / dt * 1e-12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
             "sample": f"first {sample_tokens} tokens of {wl_name} (M={wl.rows} rows, full H/F), layer0+layer1, "
-                      f"fp32 matmul on bf16-valued inputs, {dt:.2f} s wall"}
+                      f"fp32 matmul on bf16-valued inputs; 1 warm-up + {passes} timed passes, median {dt:.2f} s "
+                      f"(min {min(times):.2f}, max {max(times):.2f})"}
 
 
 def gemm_entry(t_ms, flops, peak=PEAK_BF16_TFLOPS, key="frac_bf16_peak"):
@@ -230,6 +240,17 @@ def aux_measurements(torch, capi, configs, a, wl, dev, gen, tensors):
     kernels["layer1_gemm_then_gather_reduce"] = gemm_entry(t_two, gemm_flops)
     kernels["layer1_reduce_fused_in_epilogue"] = gemm_entry(t_fused, gemm_flops)
     del z32, ws
+
+    # -- the same two GEMMs with uniform splits (rows / experts each): what the ragged routing of the workload costs --
+    if m % e == 0:
+        spu = torch.full((e,), m // e, dtype=torch.int32, device=dev)
+        giu = torch.from_numpy(wl.gather_index).to(dev)
+        z32 = torch.empty(m, h, dtype=torch.float32, device=dev)
+        kernels["gemm_layer0_uniform_splits"] = gemm_entry(time_loop(torch, lambda: capi.grouped_gemm(x, w1, spu, out=y, gather_a=giu), 20), gemm_flops)
+        kernels["gemm_layer1_uniform_splits"] = gemm_entry(time_loop(torch, lambda: capi.grouped_gemm(y, w2, spu, out=z32, row_scale=row_w), 20), gemm_flops)
+        kernels["gemm_layer0_workload_splits"] = gemm_entry(time_loop(torch, lambda: capi.grouped_gemm(x, w1, sp, out=y, gather_a=giu), 20), gemm_flops)
+        kernels["gemm_layer1_workload_splits"] = gemm_entry(time_loop(torch, lambda: capi.grouped_gemm(y, w2, sp, out=z32, row_scale=row_w), 20), gemm_flops)
+        del z32, spu
 
     # -- stand-alone HBM kernels --
     zb = torch.randn(m, h, generator=gen, device=dev).to(torch.bfloat16)
@@ -458,11 +479,20 @@ def main():
     if not a.no_aux:
         kernels.update(aux_measurements(torch, capi, configs, a, wl, dev, gen, (x, w1, w2, y, out, row_w)))
 
-    if a.calib_copy:
+    if not a.no_calib:
+        # What this box gives plain streaming kernels (the library's own copy and sum kernels, not this build's): a
+        # 1 GiB copy, copies of the byte counts the C4 / C5 reductions move, and a pure read stream of those bytes.
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
         dst = torch.empty_like(src)
         t_cp = time_loop(torch, lambda: dst.copy_(src), 5, warm=1)
-        kernels["calib_copy_1GiB"] = {"ms": round(t_cp, 4), "gbs": round(2 * (1 << 30) / t_cp * 1e-6, 1)}
+        kernels["calib_copy_1GiB"] = dict(hbm_entry(t_cp, 2 * (1 << 30)), kernel="torch copy_, 1 GiB read + 1 GiB written")
+        for tag, nbytes in (("c4", 470.6e6), ("c5", 528.7e6)):
+            nel = int(nbytes / 2) // 4                       # half read, half written
+            t_c = time_loop(torch, lambda: dst[:nel].copy_(src[:nel]), 20, warm=2)
+            kernels[f"calib_copy_reduce_bytes_{tag}"] = dict(hbm_entry(t_c, nel * 8), kernel="torch copy_")
+            nel_r = int(nbytes) // 4
+            t_r = time_loop(torch, lambda: torch.sum(src[:nel_r]), 20, warm=2)
+            kernels[f"calib_read_reduce_bytes_{tag}"] = dict(hbm_entry(t_r, nel_r * 4), kernel="torch sum (read stream)")
         del src, dst
 
     result = {

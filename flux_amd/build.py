@@ -9,6 +9,7 @@ include are compiled again.  Outputs land in flux_amd/lib/ and travel with the s
 """
 import argparse
 import concurrent.futures
+import hashlib
 import os
 import subprocess
 import sys
@@ -65,12 +66,23 @@ def _deps_of(depfile):
     return [t for t in rhs.split() if t]
 
 
-def _object_current(obj, depfile):
+def _object_current(obj, depfile, cmd):
+    """True when `obj` was built by exactly `cmd` (recorded beside the dependency file) and is newer than everything
+    it includes: a changed compiler flag rebuilds like a changed source does."""
     deps = _deps_of(depfile)
     if deps is None or not os.path.exists(obj):
         return False
+    try:
+        if open(depfile + ".cmd").read() != _cmd_stamp(cmd):
+            return False
+    except OSError:
+        return False
     t = os.path.getmtime(obj)
     return all(os.path.exists(d) and os.path.getmtime(d) <= t for d in deps)
+
+
+def _cmd_stamp(cmd):
+    return hashlib.sha256("\0".join(cmd).encode()).hexdigest()
 
 
 def build_kernels(force=True):
@@ -81,15 +93,24 @@ def build_kernels(force=True):
     def compile_one(name):
         obj = os.path.join(OBJ_DIR, name[:-4] + ".o")
         dep = obj[:-2] + ".d"
-        if not force and _object_current(obj, dep):
+        cmd = [HIPCC, *HIP_FLAGS, *EXTRA_HIP_FLAGS.get(name, []), "-MD", "-MF", dep, "-c", os.path.join(KERNEL_DIR, name), "-o", obj]
+        if not force and _object_current(obj, dep, cmd):
             return obj
-        _run([HIPCC, *HIP_FLAGS, *EXTRA_HIP_FLAGS.get(name, []), "-MD", "-MF", dep, "-c", os.path.join(KERNEL_DIR, name), "-o", obj])
+        if os.path.exists(dep + ".cmd"):
+            os.remove(dep + ".cmd")
+        _run(cmd)
+        with open(dep + ".cmd", "w") as f:
+            f.write(_cmd_stamp(cmd))
         rebuilt.append(name)
         return obj
 
     with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(srcs))) as pool:
         objs = list(pool.map(compile_one, srcs))
-    if rebuilt or not os.path.exists(KERNEL_LIB):
+    # Relink whenever an object is newer than the library (also after a link that failed: the stale library is
+    # removed first, so a failed link never leaves an old one behind).
+    if rebuilt or not os.path.exists(KERNEL_LIB) or any(os.path.getmtime(o) > os.path.getmtime(KERNEL_LIB) for o in objs):
+        if os.path.exists(KERNEL_LIB):
+            os.remove(KERNEL_LIB)
         _run([HIPCC, f"--offload-arch={ARCH}", "-shared", "-fPIC", *objs, "-o", KERNEL_LIB])
     return KERNEL_LIB
 

@@ -9,9 +9,7 @@ import os
 
 import torch
 
-# $FLUX_AMD_KERNEL_LIB names another build of the same library (an A/B comparison, a debug build).
-_LIB_PATH = os.environ.get("FLUX_AMD_KERNEL_LIB") or os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib",
-                                                                  "libfluxmi_kernels.so")
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libfluxmi_kernels.so")
 _lib = None
 
 BF16 = 0
@@ -20,7 +18,7 @@ FP8_E4M3 = 1
 EXPORTS = (
     "fluxmi_version", "fluxmi_last_error", "fluxmi_device_cu_count",
     "fluxmi_moe_route_sort_workspace_bytes", "fluxmi_moe_route_sort", "fluxmi_moe_gather_index",
-    "fluxmi_moe_route_sort_static_max_bytes", "fluxmi_moe_route_sort_static",
+    "fluxmi_moe_route_sort_static_max_bytes", "fluxmi_moe_route_sort_static_init", "fluxmi_moe_route_sort_static",
     "fluxmi_grouped_gemm_workspace_bytes", "fluxmi_grouped_gemm", "fluxmi_grouped_gemm_kernel_kind",
     "fluxmi_grouped_gemm_multi", "fluxmi_grouped_gemm_topk_reduce_workspace_bytes",
     "fluxmi_grouped_gemm_topk_reduce", "fluxmi_grouped_gemm_blockscale",

@@ -384,8 +384,13 @@ constexpr size_t kStaticScratchBytes = size_t{4} << 20;  // 4 MiB per GPU, held 
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 std::atomic<void *> g_scratch_ptr[64];  // device id -> device address of `scratch` on that GPU
+// device id -> event recorded behind the last eager call on that GPU.  The next eager call's stream waits for it, so
+// that calls issued one after the other from different streams run one after the other on the shared array instead
+// of racing.  (Host threads that call at the same moment, and replays of a captured graph against eager calls, are
+// still the caller's to order.)
+std::atomic<hipEvent_t> g_scratch_event[64];
 
-int static_scratch(void **out) {
+int static_scratch(void **out, int *dev_out) {
   int dev = 0;
   FLUXMI_HIP_CHECK(hipGetDevice(&dev));
   FLUXMI_REQUIRE(dev >= 0 && dev < 64, FLUXMI_ERR_UNSUPPORTED, "moe_route_sort_static: device id %d outside [0,64)", dev);
@@ -396,6 +401,7 @@ int static_scratch(void **out) {
     g_scratch_ptr[dev].store(ptr, std::memory_order_release);  // a lost race stores the same address
   }
   *out = ptr;
+  *dev_out = dev;
   return FLUXMI_OK;
 }
 
@@ -403,6 +409,12 @@ int static_scratch(void **out) {
 }  // namespace fluxmi
 
 extern "C" size_t fluxmi_moe_route_sort_static_max_bytes(void) { return fluxmi::kStaticScratchBytes; }
+
+extern "C" int fluxmi_moe_route_sort_static_init(void) {
+  void *ws = nullptr;
+  int dev = 0;
+  return fluxmi::static_scratch(&ws, &dev);
+}
 
 extern "C" int fluxmi_moe_route_sort_static(const int32_t *choosed, int32_t ntokens, int32_t topk,
                                             int32_t nexperts, int32_t *splits, int32_t *offsets,
@@ -417,10 +429,36 @@ extern "C" int fluxmi_moe_route_sort_static(const int32_t *choosed, int32_t ntok
                  "array holds %zu; use fluxmi_moe_route_sort with a workspace",
                  ntokens, topk, nexperts, need, kStaticScratchBytes);
   void *ws = nullptr;
-  const int rs = static_scratch(&ws);
+  int dev = 0;
+  const int rs = static_scratch(&ws, &dev);
   if (rs != FLUXMI_OK) return rs;
-  return route_sort_on_workspace(choosed, ntokens, topk, nexperts, splits, offsets, scatter_index, gather_index,
-                                 topk_index, ws, stream);
+  // Eager calls are chained through an event (created once per device: a host object, no device memory); a call
+  // on a capturing stream records nothing outside its graph and is ordered by the graph's own edges.
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  FLUXMI_HIP_CHECK(hipStreamIsCapturing(s, &cap));
+  hipEvent_t ev = nullptr;
+  if (cap == hipStreamCaptureStatusNone) {
+    ev = g_scratch_event[dev].load(std::memory_order_acquire);
+    if (ev == nullptr) {
+      hipEvent_t fresh = nullptr;
+      FLUXMI_HIP_CHECK(hipEventCreateWithFlags(&fresh, hipEventDisableTiming));
+      hipEvent_t expected = nullptr;
+      if (g_scratch_event[dev].compare_exchange_strong(expected, fresh, std::memory_order_acq_rel)) {
+        ev = fresh;
+      } else {
+        (void)hipEventDestroy(fresh);
+        ev = expected;
+      }
+    } else {
+      FLUXMI_HIP_CHECK(hipStreamWaitEvent(s, ev, 0));
+    }
+  }
+  const int rc2 = route_sort_on_workspace(choosed, ntokens, topk, nexperts, splits, offsets, scatter_index, gather_index,
+                                          topk_index, ws, stream);
+  if (rc2 != FLUXMI_OK) return rc2;
+  if (ev != nullptr) FLUXMI_HIP_CHECK(hipEventRecord(ev, s));
+  return FLUXMI_OK;
 }
 
 extern "C" int fluxmi_moe_gather_index(const int32_t *scatter_index, int32_t nrows, int32_t topk,

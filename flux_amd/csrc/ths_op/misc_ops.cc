@@ -133,11 +133,29 @@ static torch::Tensor blockscale_run(const torch::Tensor &input, const torch::Ten
   TORCH_CHECK(k % kBlock == 0, "K must be a multiple of 128, got ", k);
   FLUX_AMD_CHECK_INPUT(input_scale, at::kFloat);
   FLUX_AMD_CHECK_INPUT(weight_scale, at::kFloat);
-  const int64_t kb = k / kBlock, nb = (n + kBlock - 1) / kBlock;
-  TORCH_CHECK(weight_scale.numel() == e * nb * kb, "weight_scale has ", weight_scale.numel(), " entries, expected ",
-              e * nb * kb);
-  const int64_t want_a = a_layout == FLUXMI_ASCALE_BLOCK128 ? (m + kBlock - 1) / kBlock * kBlock * kb : m * kb;
-  TORCH_CHECK(input_scale.numel() == want_a, "input_scale has ", input_scale.numel(), " entries, expected ", want_a);
+  const int64_t kb = k / kBlock, nb = (n + kBlock - 1) / kBlock, mb = (m + kBlock - 1) / kBlock;
+  // The layout is taken from the rank, so the shape has to be exactly that layout's: a tensor of the right size in
+  // another arrangement (a [E, K/128, N/128] weight scale, a natural [M, K/128] input scale) would be read wrongly
+  // without any error.
+  if (b_layout == FLUXMI_BSCALE_N_K) {
+    TORCH_CHECK(weight_scale.dim() == 3 && weight_scale.size(0) == e && weight_scale.size(1) == nb && weight_scale.size(2) == kb,
+                "weight_scale must be a 3-D tensor [E, ceil(N/128), K/128] = [", e, ", ", nb, ", ", kb,
+                "] (as Quantization returns it) or the reference's flat 1-D [E * K/128 * N/128]; got ", weight_scale.sizes());
+  } else {
+    TORCH_CHECK(weight_scale.dim() == 1 && weight_scale.numel() == e * nb * kb,
+                "weight_scale must be a 3-D tensor [E, ceil(N/128), K/128] or the reference's flat 1-D tensor of ",
+                e * nb * kb, " entries ([E, K/128, N/128]); got ", weight_scale.sizes());
+  }
+  if (a_layout == FLUXMI_ASCALE_BLOCK128) {
+    TORCH_CHECK(input_scale.dim() == 3 && input_scale.size(0) == mb && input_scale.size(1) == kb && input_scale.size(2) == kBlock,
+                "input_scale must be a 3-D tensor [ceil(M/128), K/128, 128] = [", mb, ", ", kb, ", ", kBlock,
+                "] (as Quantization returns it) or the reference's flat 1-D tensor (per expert [K/128, M_e]); got ",
+                input_scale.sizes());
+  } else {
+    TORCH_CHECK(input_scale.dim() == 1 && input_scale.numel() == m * kb,
+                "input_scale must be a 3-D tensor [ceil(M/128), K/128, 128] or the reference's flat 1-D tensor of ", m * kb,
+                " entries (per expert [K/128, M_e], experts back to back); got ", input_scale.sizes());
+  }
   torch::Tensor out;
   if (output.has_value()) {
     out = *output;
@@ -177,8 +195,9 @@ torch::Tensor BlockScaleGemm::forward(torch::Tensor input, torch::Tensor weight,
   FLUX_AMD_CHECK_NDIM(input, 2);
   FLUX_AMD_CHECK_NDIM(weight, 2);
   torch::Tensor splits = torch::full({1}, input.size(0), at::TensorOptions().dtype(at::kInt));
-  return blockscale_run(input, weight.unsqueeze(0), splits, output, *input_scale, FLUXMI_ASCALE_BLOCK128, *weight_scale,
-                        FLUXMI_BSCALE_N_K, output_dtype_);
+  TORCH_CHECK(weight_scale->dim() == 2, "weight_scale must be [ceil(N/128), K/128], got ", weight_scale->sizes());
+  return blockscale_run(input, weight.unsqueeze(0), splits, output, *input_scale, FLUXMI_ASCALE_BLOCK128,
+                        weight_scale->unsqueeze(0), FLUXMI_BSCALE_N_K, output_dtype_);
 }
 
 torch::Tensor BlockScaleGemm::forward_grouped(torch::Tensor input, torch::Tensor input_splits, torch::Tensor weight,
@@ -194,6 +213,10 @@ torch::Tensor BlockScaleGemm::forward_grouped(torch::Tensor input, torch::Tensor
   TORCH_CHECK(input_splits.size(0) == weight.size(0), "splits 0-dim mismatch: ", input_splits.size(0), " != ",
               weight.size(0));
   TORCH_CHECK(input_splits.sum().item<int64_t>() <= input.size(0), "input_splits sum exceeds the rows of input");
+  TORCH_CHECK(input_scale.dim() == 3 || input_scale.dim() == 1, "input_scale must be 3-D [ceil(M/128), K/128, 128] or the "
+              "reference's flat 1-D layout (per expert [K/128, M_e]); got ", input_scale.sizes());
+  TORCH_CHECK(weight_scale.dim() == 3 || weight_scale.dim() == 1, "weight_scale must be 3-D [E, ceil(N/128), K/128] or the "
+              "reference's flat 1-D layout ([E, K/128, N/128]); got ", weight_scale.sizes());
   const int32_t a_layout = input_scale.dim() == 3 ? FLUXMI_ASCALE_BLOCK128 : FLUXMI_ASCALE_EXPERT_K_M;
   const int32_t b_layout = weight_scale.dim() == 3 ? FLUXMI_BSCALE_N_K : FLUXMI_BSCALE_K_N;
   return blockscale_run(input, weight, input_splits, output, input_scale, a_layout, weight_scale, b_layout, output_dtype_);

@@ -111,8 +111,8 @@ PYBIND11_MODULE(flux_ths_pybind, m) {
       .def(py::init<torch::Tensor, int64_t>(), py::arg("weight"), py::arg("num_experts"))
       .def("forward", &GemmGroupedV3::forward, py::arg("input"), py::arg("splits_cpu"));
 
-  // src/pybind/gemm_only.cc:77-139 (forward and forward_grouped; the weight-gradient and multi-stream methods are
-  // not built)
+  // src/pybind/gemm_only.cc:77-139 (forward, forward_grouped, forward_multistream, reference, profiling; only the
+  // weight-gradient methods wgrad* are absent)
   py::class_<BlockScaleGemm>(m, "BlockScaleGemm")
       .def(py::init([](py::object input_dtype, py::object weight_dtype, py::object output_dtype, int32_t num_streams) {
              const at::ScalarType in = to_dtype(input_dtype);

@@ -89,8 +89,8 @@ class GemmGroupedV3 {
 };
 
 // Block-scaled fp8 GEMM of the reference (src/comm_none/ths_op/blockscale_gemm.h:24-94): the forward
-// products, dense and grouped.  wgrad / the multi-stream variants (training-time weight gradients, per-expert
-// streams) are not on this path and are not built.
+// products, dense and grouped (forward_multistream is the same single launch).  The wgrad* methods (training-time
+// weight gradients) are not on this path and are not built.
 class BlockScaleGemm {
  public:
   BlockScaleGemm(at::ScalarType input_dtype, at::ScalarType weight_dtype, at::ScalarType output_dtype,

@@ -66,9 +66,14 @@ int fluxmi_moe_route_sort(const int32_t *choosed, int32_t ntokens, int32_t topk,
  * the process ends); the call itself allocates and frees nothing.  Inputs whose
  * fluxmi_moe_route_sort_workspace_bytes() exceeds that size are rejected with FLUXMI_ERR_WORKSPACE (the limit
  * is (ceil(ntokens*topk / 512) + 1) * nexperts <= 1048576).  All calls on one GPU share the one array: calls
- * that overlap in time on the same GPU (different streams or threads) race; calls on one stream are ordered.
- * Results are bit-identical to fluxmi_moe_route_sort. */
+ * on one stream are ordered, and eager calls issued one after the other from different streams are chained by an
+ * event the library keeps per GPU; calls issued at the same moment from several host threads, and replays of a
+ * captured graph against other calls, are the caller's to order: they race on the array and give wrong indices.
+ * fluxmi_moe_route_sort_static_init() looks up the array's device address for the current device (the only set-up
+ * there is); the first call on a device does the same, so a caller whose first call would be under stream capture
+ * calls the init function beforehand, outside the capture.  Results are bit-identical to fluxmi_moe_route_sort. */
 size_t fluxmi_moe_route_sort_static_max_bytes(void);
+int fluxmi_moe_route_sort_static_init(void);
 int fluxmi_moe_route_sort_static(const int32_t *choosed, int32_t ntokens, int32_t topk, int32_t nexperts,
                                  int32_t *splits, int32_t *offsets, int32_t *scatter_index,
                                  int32_t *gather_index, int32_t *topk_index, void *stream);

@@ -365,6 +365,14 @@ def test_blockscale_gemm_op_dense_and_grouped():
         op.forward(qx, qw[0], bias=torch.zeros(1, device="cuda"), input_scale=sx, weight_scale=sw[0].contiguous())
     with pytest.raises(RuntimeError, match="cpu"):
         op.forward_grouped(qx, torch.from_numpy(split).cuda(), qw, input_scale=sx, weight_scale=sw)
+    # scales of the right size in another arrangement are rejected instead of being read in the wrong layout
+    assert n // 128 != k // 128
+    with pytest.raises(RuntimeError, match="weight_scale must be"):
+        op.forward_grouped(qx, torch.from_numpy(split), qw, input_scale=sx, weight_scale=sw.transpose(1, 2).contiguous())
+    with pytest.raises(RuntimeError, match="input_scale must be"):
+        op.forward_grouped(qx, torch.from_numpy(split), qw, input_scale=sa.contiguous().cuda(), weight_scale=sw)
+    with pytest.raises(RuntimeError, match="input_scale must be"):
+        op.forward(qx, qw[0], input_scale=sx.reshape(-1), weight_scale=sw[0].contiguous())
 
 
 def test_layer1_op_with_the_fused_epilogue_reduce(c1, monkeypatch):

@@ -20,6 +20,7 @@ def _outputs(tokens, topk, experts, dev):
 def test_static_scratch_route_sort_equals_workspace_route_sort_twice():
     from flux_amd import capi
     dev = torch.device("cuda:0")
+    assert capi.load().fluxmi_moe_route_sort_static_init() == 0  # the set-up a caller does ahead of a capture
     first = True
     # a large three-kernel case, then smaller ones (two-kernel and single-workgroup paths) on the same scratch
     for name, tokens in (("C4", 40000), ("C4", None), ("C3", None), ("C5", 300), ("C1", None)):
@@ -28,10 +29,13 @@ def test_static_scratch_route_sort_equals_workspace_route_sort_twice():
         choosed = wl.choosed.to(dev)
         out = _outputs(wl.tokens, wl.topk, wl.experts, dev)
         torch.cuda.synchronize()
-        before = torch.cuda.memory_allocated()
+        # torch's allocator only sees torch's own requests; the device's free memory (hipMemGetInfo) also sees a
+        # hipMalloc / hipFree made inside the library
+        before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
         capi.route_sort_static(choosed, wl.experts, out)
         torch.cuda.synchronize()
         assert torch.cuda.memory_allocated() == before
+        assert torch.cuda.mem_get_info()[0] == free_before, "device memory changed hands during the call"
         ref = capi.route_sort(choosed, wl.experts)
         for got, want, nm in zip(out, ref, ("splits", "offsets", "scatter_index", "gather_index", "topk_index")):
             assert torch.equal(got, want), f"{name}: {nm} differs from fluxmi_moe_route_sort"
