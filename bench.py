@@ -480,19 +480,21 @@ def main():
         kernels.update(aux_measurements(torch, capi, configs, a, wl, dev, gen, (x, w1, w2, y, out, row_w)))
 
     if not a.no_calib:
-        # What this box gives plain streaming kernels (the library's own copy and sum kernels, not this build's): a
-        # 1 GiB copy, copies of the byte counts the C4 / C5 reductions move, and a pure read stream of those bytes.
+        # What this box gives kernels that only stream (fluxmi_calib_stream: 16 bytes per lane and load, eight loads in
+        # flight, non-temporal): a 1 GiB copy (also the known traffic that scales the profiler's byte counters), and,
+        # for the byte counts the C4 / C5 reductions and the quantisation shapes move, a copy and a pure read stream.
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
         dst = torch.empty_like(src)
-        t_cp = time_loop(torch, lambda: dst.copy_(src), 5, warm=1)
-        kernels["calib_copy_1GiB"] = dict(hbm_entry(t_cp, 2 * (1 << 30)), kernel="torch copy_, 1 GiB read + 1 GiB written")
-        for tag, nbytes in (("c4", 470.6e6), ("c5", 528.7e6)):
-            nel = int(nbytes / 2) // 4                       # half read, half written
-            t_c = time_loop(torch, lambda: dst[:nel].copy_(src[:nel]), 20, warm=2)
-            kernels[f"calib_copy_reduce_bytes_{tag}"] = dict(hbm_entry(t_c, nel * 8), kernel="torch copy_")
-            nel_r = int(nbytes) // 4
-            t_r = time_loop(torch, lambda: torch.sum(src[:nel_r]), 20, warm=2)
-            kernels[f"calib_read_reduce_bytes_{tag}"] = dict(hbm_entry(t_r, nel_r * 4), kernel="torch sum (read stream)")
+        t_cp = time_loop(torch, lambda: capi.calib_stream(src, dst, 1 << 30, copy=True), 5, warm=1)
+        kernels["calib_copy_1GiB"] = dict(hbm_entry(t_cp, 2 * (1 << 30)), kernel="plain copy, 1 GiB read + 1 GiB written")
+        t_tc = time_loop(torch, lambda: dst.copy_(src), 5, warm=1)
+        kernels["calib_copy_1GiB_library"] = dict(hbm_entry(t_tc, 2 * (1 << 30)), kernel="torch copy_")
+        for tag, nbytes in (("reduce_c4", 470.6e6), ("reduce_c5", 528.7e6), ("quant_4096x7168", 88.1e6)):
+            nb = int(nbytes) // 32 * 32
+            t_c = time_loop(torch, lambda: capi.calib_stream(src, dst, nb // 2, copy=True), 20, warm=2)
+            kernels[f"calib_copy_bytes_of_{tag}"] = dict(hbm_entry(t_c, nb), kernel="plain copy, half read, half written")
+            t_r = time_loop(torch, lambda: capi.calib_stream(src, dst, nb, copy=False), 20, warm=2)
+            kernels[f"calib_read_bytes_of_{tag}"] = dict(hbm_entry(t_r, nb), kernel="plain read stream")
         del src, dst
 
     result = {

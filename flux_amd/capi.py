@@ -14,6 +14,14 @@ _lib = None
 
 BF16 = 0
 FP8_E4M3 = 1
+FP16 = 2
+_DTYPES = {torch.bfloat16: BF16, torch.float8_e4m3fn: FP8_E4M3, torch.float16: FP16}
+
+
+def _half_out(in_dtype):
+    """16-bit output type of an operand type: fp16 operands give fp16, bf16 and fp8 give bf16."""
+    return torch.float16 if in_dtype == torch.float16 else torch.bfloat16
+
 
 EXPORTS = (
     "fluxmi_version", "fluxmi_last_error", "fluxmi_device_cu_count",
@@ -23,7 +31,7 @@ EXPORTS = (
     "fluxmi_grouped_gemm_multi", "fluxmi_grouped_gemm_topk_reduce_workspace_bytes",
     "fluxmi_grouped_gemm_topk_reduce", "fluxmi_grouped_gemm_blockscale",
     "fluxmi_topk_gather_reduce", "fluxmi_quant_e4m3_rowwise", "fluxmi_quant_e4m3_square",
-    "fluxmi_quant_e4m3_block128",
+    "fluxmi_quant_e4m3_block128", "fluxmi_calib_stream_sink_bytes", "fluxmi_calib_stream",
 )
 
 
@@ -77,6 +85,8 @@ def load():
     lib.fluxmi_quant_e4m3_rowwise.argtypes = [vp, i64, i64, i32, f32, vp, vp, i32, vp]
     lib.fluxmi_quant_e4m3_square.argtypes = [vp, i64, i64, i64, f32, vp, vp, vp, vp, vp]
     lib.fluxmi_quant_e4m3_block128.argtypes = [vp, i64, i64, f32, vp, vp, vp, vp, vp]
+    lib.fluxmi_calib_stream_sink_bytes.restype = sz
+    lib.fluxmi_calib_stream.argtypes = [vp, vp, sz, i32, vp]
     _lib = lib
     return lib
 
@@ -150,15 +160,14 @@ def gather_index(scatter_index, topk):
 
 SCHED_WHOLE_TAIL_TILES = 1
 SCHED_NO_HALF_TILES = 2
+SCHED_NO_SKINNY_TAIL = 4
+SCHED_FORCE_SKINNY_TAIL = 8
 
 
 def _gemm_args(a, b, splits, out, gather_a, scatter_d, alpha, row_scale, col_scale, scalar_scale, scalar_scale_dev,
                max_rows, out_dtype, cu_margin, raster_rows, sched_flags, need_out=True):
-    if a.dtype == torch.bfloat16:
-        dtype = BF16
-    elif a.dtype == torch.float8_e4m3fn:
-        dtype = FP8_E4M3
-    else:
+    dtype = _DTYPES.get(a.dtype)
+    if dtype is None:
         raise ValueError(f"unsupported input dtype {a.dtype}")
     _dev_tensor(a, a.dtype, "a")
     _dev_tensor(b, a.dtype, "b")
@@ -175,9 +184,9 @@ def _gemm_args(a, b, splits, out, gather_a, scatter_d, alpha, row_scale, col_sca
         max_rows = gather_a.numel() if gather_a is not None else a.shape[0]
     if need_out:
         if out is None:
-            out = torch.empty(max_rows, n, dtype=out_dtype or torch.bfloat16, device=a.device)
-        if out.dtype not in (torch.bfloat16, torch.float32):
-            raise ValueError(f"out must be bf16 or fp32, got {out.dtype}")
+            out = torch.empty(max_rows, n, dtype=out_dtype or _half_out(a.dtype), device=a.device)
+        if out.dtype not in (_half_out(a.dtype), torch.float32):
+            raise ValueError(f"out must be {_half_out(a.dtype)} or fp32, got {out.dtype}")
         _dev_tensor(out, out.dtype, "out")
         if out.shape[0] < max_rows or out.shape[1] != n:
             raise ValueError(f"out {tuple(out.shape)} too small for [{max_rows}, {n}]")
@@ -238,8 +247,8 @@ def grouped_gemm_topk_reduce(a, b, splits, token_of_row, ntokens, out=None, work
                          scalar_scale_dev, max_rows, None, 0, 0, 0, need_out=False)
     n = b.shape[1]
     if out is None:
-        out = torch.empty(ntokens, n, dtype=torch.bfloat16, device=a.device)
-    _dev_tensor(out, torch.bfloat16, "out")
+        out = torch.empty(ntokens, n, dtype=_half_out(a.dtype), device=a.device)
+    _dev_tensor(out, _half_out(a.dtype), "out")
     ws_bytes = lib.fluxmi_grouped_gemm_topk_reduce_workspace_bytes(ntokens, n)
     if workspace is None:
         workspace = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=a.device)
@@ -250,11 +259,11 @@ def grouped_gemm_topk_reduce(a, b, splits, token_of_row, ntokens, out=None, work
 
 
 def grouped_gemm_multi(a, bs, splits, outs=None, gather_a=None, alphas=None, row_scale=None, col_scale=None,
-                       scalar_scale=1.0, max_rows=None, out_dtype=None):
+                       scalar_scale=1.0, max_rows=None, out_dtype=None, raster_rows=0, sched_flags=0):
     """[A @ B_g for B_g in bs] in one launch (fluxmi_grouped_gemm_multi): the same sorted rows times up to four
     weight tensors [E, N, K], each with its own output and optional per-expert alpha."""
     lib = load()
-    dtype = {torch.bfloat16: BF16, torch.float8_e4m3fn: FP8_E4M3}.get(a.dtype)
+    dtype = _DTYPES.get(a.dtype)
     if dtype is None:
         raise ValueError(f"unsupported input dtype {a.dtype}")
     ng = len(bs)
@@ -273,10 +282,10 @@ def grouped_gemm_multi(a, bs, splits, outs=None, gather_a=None, alphas=None, row
     if max_rows is None:
         max_rows = gather_a.numel() if gather_a is not None else a.shape[0]
     if outs is None:
-        outs = [torch.empty(max_rows, n, dtype=out_dtype or torch.bfloat16, device=a.device) for _ in range(ng)]
+        outs = [torch.empty(max_rows, n, dtype=out_dtype or _half_out(a.dtype), device=a.device) for _ in range(ng)]
     for o in outs:
         _dev_tensor(o, outs[0].dtype, "out")
-        if o.dtype not in (torch.bfloat16, torch.float32) or o.shape[0] < max_rows or o.shape[1] != n:
+        if o.dtype not in (_half_out(a.dtype), torch.float32) or o.shape[0] < max_rows or o.shape[1] != n:
             raise ValueError(f"out {tuple(o.shape)} {o.dtype} does not fit [{max_rows}, {n}] bf16/fp32")
     if len(outs) != ng or (alphas is not None and len(alphas) != ng):
         raise ValueError("outs / alphas need one entry per weight group")
@@ -287,7 +296,8 @@ def grouped_gemm_multi(a, bs, splits, outs=None, gather_a=None, alphas=None, row
         splits=splits.data_ptr(), gather_a=None if gather_a is None else gather_a.data_ptr(), scatter_d=None,
         alpha=None, row_scale=None if row_scale is None else row_scale.data_ptr(),
         col_scale=None if col_scale is None else col_scale.data_ptr(), scalar_scale=float(scalar_scale),
-        d_fp32=int(outs[0].dtype == torch.float32), scalar_scale_dev=None)
+        d_fp32=int(outs[0].dtype == torch.float32), scalar_scale_dev=None, raster_rows=raster_rows,
+        sched_flags=sched_flags)
     vps = ctypes.c_void_p * ng
     b_arr = vps(*[b.data_ptr() for b in bs])
     d_arr = vps(*[o.data_ptr() for o in outs])
@@ -297,14 +307,15 @@ def grouped_gemm_multi(a, bs, splits, outs=None, gather_a=None, alphas=None, row
     return outs
 
 
-def topk_gather_reduce(inputs, routing_idx, topk, row_weight=None, scale=1.0, out=None):
-    """out[t] = bf16(scale * sum_g sum_j w[r] * inputs[g][r]), r = routing_idx[t*topk+j]."""
+def topk_gather_reduce(inputs, routing_idx, topk, row_weight=None, scale=1.0, out=None, out_dtype=None):
+    """out[t] = bf16(scale * sum_g sum_j w[r] * inputs[g][r]), r = routing_idx[t*topk+j].  fp16 inputs give an fp16
+    result; fp32 inputs give bf16 unless out / out_dtype say fp16."""
     lib = load()
     if isinstance(inputs, torch.Tensor):
         inputs = [inputs]
     in_dtype = inputs[0].dtype
-    if in_dtype not in (torch.bfloat16, torch.float32):
-        raise ValueError(f"inputs must be bf16 or fp32, got {in_dtype}")
+    if in_dtype not in (torch.bfloat16, torch.float32, torch.float16):
+        raise ValueError(f"inputs must be bf16, fp16 or fp32, got {in_dtype}")
     for g, t in enumerate(inputs):
         _dev_tensor(t, in_dtype, f"inputs[{g}]")
     _dev_tensor(routing_idx, torch.int32, "routing_idx")
@@ -314,9 +325,12 @@ def topk_gather_reduce(inputs, routing_idx, topk, row_weight=None, scale=1.0, ou
         raise ValueError("routing_idx length is not a multiple of topk")
     ntokens = routing_idx.numel() // topk
     if out is None:
-        out = torch.empty(ntokens, n, dtype=torch.bfloat16, device=inputs[0].device)
+        out = torch.empty(ntokens, n, dtype=out_dtype or _half_out(in_dtype), device=inputs[0].device)
+    if out.dtype != (_half_out(in_dtype) if in_dtype != torch.float32 else out.dtype) or out.dtype not in (torch.bfloat16, torch.float16):
+        raise ValueError(f"out dtype {out.dtype} does not go with {in_dtype} inputs")
+    io_format = int(in_dtype == torch.float32) | (2 if out.dtype == torch.float16 else 0)
     ptrs = (ctypes.c_void_p * len(inputs))(*[t.data_ptr() for t in inputs])
-    _check(lib.fluxmi_topk_gather_reduce(ptrs, len(inputs), int(in_dtype == torch.float32), _ptr(routing_idx), _ptr(row_weight),
+    _check(lib.fluxmi_topk_gather_reduce(ptrs, len(inputs), io_format, _ptr(routing_idx), _ptr(row_weight),
                                          float(scale), ntokens, topk, n, _ptr(out), _stream()),
            "fluxmi_topk_gather_reduce")
     return out
@@ -394,3 +408,13 @@ def quant_e4m3_block128(x, eps=0.0, transpose=False):
     _check(lib.fluxmi_quant_e4m3_block128(_ptr(x), rows, cols, float(eps), _ptr(q), _ptr(si), _ptr(qt), _ptr(sit),
                                           _stream()), "fluxmi_quant_e4m3_block128")
     return q, si, qt, sit
+
+
+def calib_stream(src, dst, nbytes, copy=False):
+    """fluxmi_calib_stream: a plain read stream of src[:nbytes] (copy=False; dst is a small sink of at least
+    calib_stream_sink_bytes()) or a copy of it into dst."""
+    lib = load()
+    need = nbytes if copy else lib.fluxmi_calib_stream_sink_bytes()
+    if src.numel() * src.element_size() < nbytes or dst.numel() * dst.element_size() < need:
+        raise ValueError("calib_stream: buffers smaller than the stream")
+    _check(lib.fluxmi_calib_stream(_ptr(src), _ptr(dst), nbytes, int(copy), _stream()), "fluxmi_calib_stream")

@@ -75,6 +75,15 @@ __device__ __forceinline__ float bf16_bits_to_float(uint16_t b) {
   return __uint_as_float(static_cast<uint32_t>(b) << 16);
 }
 
+__device__ __forceinline__ float f16_bits_to_float(uint16_t b) {
+  return static_cast<float>(__builtin_bit_cast(_Float16, b));
+}
+
+// fp32 -> fp16 bits, round to nearest even (v_cvt_f16_f32).
+__device__ __forceinline__ uint16_t float_to_f16_bits(float f) {
+  return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f));
+}
+
 // fp32 -> bf16 bits, round to nearest even, NaN kept quiet.
 __device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
   uint32_t u = __float_as_uint(f);

@@ -56,13 +56,23 @@ __device__ __forceinline__ Vec8<IN_F32> zero8() {
   return r;
 }
 
-__device__ __forceinline__ void accumulate8(float (&acc)[8], const Vec8<true> &x, const float w) {
+// f16 (wave-uniform): 16-bit inputs are fp16 instead of bf16; fp32 inputs ignore it.
+__device__ __forceinline__ void accumulate8(float (&acc)[8], const Vec8<true> &x, const float w, bool) {
 #pragma unroll
   for (int i = 0; i < 8; ++i) acc[i] = fmaf(w, __uint_as_float(x.v[i >> 2][i & 3]), acc[i]);
 }
 
-__device__ __forceinline__ void accumulate8(float (&acc)[8], const Vec8<false> &x, const float w) {
+__device__ __forceinline__ void accumulate8(float (&acc)[8], const Vec8<false> &x, const float w, bool f16) {
   const u32x4 v = x.v[0];
+  if (f16) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t u = v[i];
+      acc[2 * i] = fmaf(w, f16_bits_to_float(static_cast<uint16_t>(u & 0xffffu)), acc[2 * i]);
+      acc[2 * i + 1] = fmaf(w, f16_bits_to_float(static_cast<uint16_t>(u >> 16)), acc[2 * i + 1]);
+    }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const uint32_t u = v[i];
@@ -77,7 +87,9 @@ __device__ __forceinline__ bool row_in_range(int32_t r, int32_t nrows) {
   return static_cast<uint32_t>(r) < static_cast<uint32_t>(nrows);
 }
 
-__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+// Two results to the packed 16-bit output type: bf16, or fp16 when f16 (wave-uniform) is set.
+__device__ __forceinline__ uint32_t pack2(float lo, float hi, bool f16) {
+  if (f16) return static_cast<uint32_t>(float_to_f16_bits(lo)) | (static_cast<uint32_t>(float_to_f16_bits(hi)) << 16);
   return static_cast<uint32_t>(float_to_bf16_bits(lo)) | (static_cast<uint32_t>(float_to_bf16_bits(hi)) << 16);
 }
 
@@ -87,7 +99,7 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
 template <int TOPK, int NGROUPS, bool WEIGHTED, bool IN_F32, bool NT>
 __device__ __forceinline__ void topk_gather_reduce_body(
     const GroupPtrs &in, const int32_t *__restrict__ routing_idx, const float *__restrict__ row_weight,
-    float scale, int32_t topk_rt, int32_t nvec, int32_t nrows, uint16_t *__restrict__ out) {
+    float scale, int32_t topk_rt, int32_t nvec, int32_t nrows, bool f16, uint16_t *__restrict__ out) {
   const int t = blockIdx.x;
   const int topk = TOPK > 0 ? TOPK : topk_rt;
   const size_t row_vecs = static_cast<size_t>(nvec);
@@ -132,14 +144,14 @@ __device__ __forceinline__ void topk_gather_reduce_body(
       u32x2 *dst = reinterpret_cast<u32x2 *>(out) + static_cast<size_t>(t) * nq;
       if (oka) {
         u32x2 o;
-        o[0] = pack2(a[0] * scale, a[1] * scale);
-        o[1] = pack2(a[2] * scale, a[3] * scale);
+        o[0] = pack2(a[0] * scale, a[1] * scale, f16);
+        o[1] = pack2(a[2] * scale, a[3] * scale, f16);
         __builtin_nontemporal_store(o, dst + qa);
       }
       if (okb) {
         u32x2 o;
-        o[0] = pack2(b[0] * scale, b[1] * scale);
-        o[1] = pack2(b[2] * scale, b[3] * scale);
+        o[0] = pack2(b[0] * scale, b[1] * scale, f16);
+        o[1] = pack2(b[2] * scale, b[3] * scale, f16);
         __builtin_nontemporal_store(o, dst + qb);
       }
     }
@@ -166,7 +178,7 @@ __device__ __forceinline__ void topk_gather_reduce_body(
 #pragma unroll
       for (int g = 0; g < NGROUPS; ++g) {
 #pragma unroll
-        for (int j = 0; j < TOPK; ++j) accumulate8(acc, vals[g][j], w[j]);
+        for (int j = 0; j < TOPK; ++j) accumulate8(acc, vals[g][j], w[j], f16);
       }
     } else {
       for (int g = 0; g < NGROUPS; ++g) {
@@ -174,17 +186,13 @@ __device__ __forceinline__ void topk_gather_reduce_body(
           const int32_t r = routing_idx[static_cast<size_t>(t) * topk + j];
           if (!row_in_range(r, nrows)) continue;
           const float w = WEIGHTED ? row_weight[r] : 1.f;
-          accumulate8(acc, load8<IN_F32, NT>(in.p[g], static_cast<size_t>(r), row_vecs, v), w);
+          accumulate8(acc, load8<IN_F32, NT>(in.p[g], static_cast<size_t>(r), row_vecs, v), w, f16);
         }
       }
     }
     u32x4 o;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const uint32_t lo = float_to_bf16_bits(acc[2 * i] * scale);
-      const uint32_t hi = float_to_bf16_bits(acc[2 * i + 1] * scale);
-      o[i] = lo | (hi << 16);
-    }
+    for (int i = 0; i < 4; ++i) o[i] = pack2(acc[2 * i] * scale, acc[2 * i + 1] * scale, f16);
     u32x4 *dst = reinterpret_cast<u32x4 *>(out) + static_cast<size_t>(t) * row_vecs + v;
     __builtin_nontemporal_store(o, dst);
   }
@@ -193,14 +201,15 @@ __device__ __forceinline__ void topk_gather_reduce_body(
 template <int TOPK, int NGROUPS, bool WEIGHTED, bool IN_F32>
 __global__ __launch_bounds__(kMaxThreads) void topk_gather_reduce_kernel(
     GroupPtrs in, const int32_t *__restrict__ routing_idx, const float *__restrict__ row_weight,
-    float scale, int32_t topk_rt, int32_t nvec /* n / 8 */, int32_t nrows, int32_t nt_loads,
+    float scale, int32_t topk_rt, int32_t nvec /* n / 8 */, int32_t nrows, int32_t flags /* 1: non-temporal loads, 2: fp16 */,
     uint16_t *__restrict__ out) {
-  if (nt_loads)
+  const bool f16 = (flags & 2) != 0;
+  if (flags & 1)
     topk_gather_reduce_body<TOPK, NGROUPS, WEIGHTED, IN_F32, true>(in, routing_idx, row_weight, scale, topk_rt,
-                                                                   nvec, nrows, out);
+                                                                   nvec, nrows, f16, out);
   else
     topk_gather_reduce_body<TOPK, NGROUPS, WEIGHTED, IN_F32, false>(in, routing_idx, row_weight, scale, topk_rt,
-                                                                    nvec, nrows, out);
+                                                                    nvec, nrows, f16, out);
 }
 
 template <int TOPK, int NGROUPS>
@@ -235,13 +244,17 @@ void dispatch_topk(bool weighted, bool in_f32, dim3 grid, int threads, int nt, h
 }  // namespace
 }  // namespace fluxmi
 
-extern "C" int fluxmi_topk_gather_reduce(const void *const *in, int32_t ngroups, int32_t in_fp32,
+extern "C" int fluxmi_topk_gather_reduce(const void *const *in, int32_t ngroups, int32_t io_format,
                                          const int32_t *routing_idx, const float *row_weight,
                                          float scale, int32_t ntokens, int32_t topk, int32_t n,
                                          void *out, void *stream) {
   using namespace fluxmi;
   FLUXMI_REQUIRE(in != nullptr && routing_idx != nullptr && out != nullptr, FLUXMI_ERR_INVALID_ARG,
                  "topk_gather_reduce: null pointer argument");
+  FLUXMI_REQUIRE(io_format >= 0 && io_format <= 3, FLUXMI_ERR_INVALID_ARG,
+                 "topk_gather_reduce: io_format=%d outside [0,3]", io_format);
+  const int32_t in_fp32 = io_format & 1;
+  const int32_t half_f16 = (io_format & 2) ? 2 : 0;
   FLUXMI_REQUIRE(ngroups >= 1 && ngroups <= kMaxGroups, FLUXMI_ERR_UNSUPPORTED,
                  "topk_gather_reduce: ngroups=%d outside [1,%d]", ngroups, kMaxGroups);
   FLUXMI_REQUIRE(topk >= 1 && topk <= 64, FLUXMI_ERR_UNSUPPORTED,
@@ -273,7 +286,7 @@ extern "C" int fluxmi_topk_gather_reduce(const void *const *in, int32_t ngroups,
     if (ysplit > 16) ysplit = 16;
   }
   const size_t in_bytes = static_cast<size_t>(ntokens) * topk * n * (in_fp32 ? 4 : 2) * ngroups;
-  const int nt = in_bytes > kPlainLoadMaxBytes ? 1 : 0;
+  const int nt = (in_bytes > kPlainLoadMaxBytes ? 1 : 0) | half_f16;
   const dim3 grid(static_cast<unsigned>(ntokens), static_cast<unsigned>(ysplit));
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool weighted = row_weight != nullptr;

@@ -52,8 +52,9 @@ __global__ __launch_bounds__(256) void grouped_gemm_generic_kernel(const GemmPar
     for (int kk = 0; kk < p.k; ++kk) {
       float av, bv;
       if (ELT == 2) {
-        av = bf16_bits_to_float(reinterpret_cast<const uint16_t *>(ap)[kk]);
-        bv = bf16_bits_to_float(reinterpret_cast<const uint16_t *>(bp)[kk]);
+        const uint16_t ab = reinterpret_cast<const uint16_t *>(ap)[kk], bb = reinterpret_cast<const uint16_t *>(bp)[kk];
+        av = p.half_is_f16 ? f16_bits_to_float(ab) : bf16_bits_to_float(ab);
+        bv = p.half_is_f16 ? f16_bits_to_float(bb) : bf16_bits_to_float(bb);
       } else {
         av = e4m3_to_float(ap[kk]);
         bv = e4m3_to_float(bp[kk]);
@@ -82,7 +83,7 @@ __global__ __launch_bounds__(256) void grouped_gemm_generic_kernel(const GemmPar
     }
     if (p.accumulate) unsafeAtomicAdd(static_cast<float *>(p.d[g]) + drow * p.n + n, v);
     else if (p.d_fp32) static_cast<float *>(p.d[g])[drow * p.n + n] = v;
-    else static_cast<uint16_t *>(p.d[g])[drow * p.n + n] = float_to_bf16_bits(v);
+    else static_cast<uint16_t *>(p.d[g])[drow * p.n + n] = p.half_is_f16 ? float_to_f16_bits(v) : float_to_bf16_bits(v);
   }
 }
 
@@ -91,7 +92,7 @@ __global__ __launch_bounds__(256) void grouped_gemm_generic_kernel(const GemmPar
 // whole, which needs its extent a_rows; 256 rows of an ungathered A; one expert's weights).  Everything else
 // runs the generic kernel.
 bool mfma_path_ok(const fluxmi_grouped_gemm_args *a, const void *b, const void *d, bool d_is_fp32) {
-  const int elt = a->dtype == FLUXMI_BF16 ? 2 : 1;
+  const int elt = a->dtype == FLUXMI_FP8_E4M3 ? 1 : 2;
   const int64_t kbytes = static_cast<int64_t>(a->k) * elt;
   const int64_t span = 0xffffffffll;
   const bool a_fits = a->gather_a ? (a->a_rows > 0 && a->a_rows * kbytes <= span) : BM * kbytes <= span;
@@ -119,7 +120,7 @@ int run_grouped_gemm(const fluxmi_grouped_gemm_args *args, int ngroups, const vo
                      const float *const *alpha, void *stream, bool dry_run = false, int32_t accumulate_rows = 0,
                      const BlockScales *bs = nullptr) {
   FLUXMI_REQUIRE(args != nullptr, FLUXMI_ERR_INVALID_ARG, "grouped_gemm: null args");
-  FLUXMI_REQUIRE(args->dtype == FLUXMI_BF16 || args->dtype == FLUXMI_FP8_E4M3, FLUXMI_ERR_INVALID_ARG,
+  FLUXMI_REQUIRE(args->dtype == FLUXMI_BF16 || args->dtype == FLUXMI_FP8_E4M3 || args->dtype == FLUXMI_FP16, FLUXMI_ERR_INVALID_ARG,
                  "grouped_gemm: unknown dtype %d", args->dtype);
   FLUXMI_REQUIRE(args->d_fp32 == 0 || args->d_fp32 == 1, FLUXMI_ERR_INVALID_ARG,
                  "grouped_gemm: d_fp32 must be 0 or 1");
@@ -166,6 +167,7 @@ int run_grouped_gemm(const fluxmi_grouped_gemm_args *args, int ngroups, const vo
   p.accumulate = accumulate_rows > 0 ? 1 : 0;
   p.d_rows = accumulate_rows > 0 ? accumulate_rows : args->max_rows;
   p.ngroups = ngroups;
+  p.half_is_f16 = args->dtype == FLUXMI_FP16 ? 1 : 0;
   p.a_scale = bs ? bs->a_scale : nullptr;
   p.b_scale = bs ? bs->b_scale : nullptr;
   p.a_scale_layout = bs ? bs->a_layout : 0;
@@ -189,7 +191,8 @@ int run_grouped_gemm(const fluxmi_grouped_gemm_args *args, int ngroups, const vo
   FLUXMI_REQUIRE(args->raster_rows >= 0 && args->raster_rows <= 1024, FLUXMI_ERR_INVALID_ARG,
                  "grouped_gemm: raster_rows=%d outside [0,1024]", args->raster_rows);
   FLUXMI_REQUIRE(args->cu_margin >= 0, FLUXMI_ERR_INVALID_ARG, "grouped_gemm: negative cu_margin");
-  FLUXMI_REQUIRE((args->sched_flags & ~(FLUXMI_SCHED_WHOLE_TAIL_TILES | FLUXMI_SCHED_NO_HALF_TILES)) == 0,
+  FLUXMI_REQUIRE((args->sched_flags & ~(FLUXMI_SCHED_WHOLE_TAIL_TILES | FLUXMI_SCHED_NO_HALF_TILES |
+                                        FLUXMI_SCHED_NO_SKINNY_TAIL | FLUXMI_SCHED_FORCE_SKINNY_TAIL)) == 0,
                  FLUXMI_ERR_INVALID_ARG, "grouped_gemm: unknown sched_flags 0x%x", args->sched_flags);
   // fp32 outputs beyond half a GB go out non-temporally (measured on a 805 MB intermediate: the GEMM 5 % faster,
   // the reduce that reads it unchanged; at 268 MB the GEMM is unchanged and the reduce 10 % slower).
@@ -210,13 +213,14 @@ int run_grouped_gemm(const fluxmi_grouped_gemm_args *args, int ngroups, const vo
     const int64_t max_tiles = (static_cast<int64_t>(args->max_rows) / BM + args->nexperts) * tiles_n;
     const int grid = static_cast<int>(max_tiles < cus ? max_tiles : cus);
     const int rc = bs != nullptr ? launch_grouped_gemm_fp8_blockscale(p, grid, s)
-                                 : (args->dtype == FLUXMI_BF16 ? launch_grouped_gemm_bf16(p, grid, s)
-                                                               : launch_grouped_gemm_fp8(p, grid, s));
+                   : args->dtype == FLUXMI_BF16 ? launch_grouped_gemm_bf16(p, grid, s)
+                   : args->dtype == FLUXMI_FP16 ? launch_grouped_gemm_f16(p, grid, s)
+                                                : launch_grouped_gemm_fp8(p, grid, s);
     if (rc != FLUXMI_OK) return rc;
   } else {
     const int grid = cus * 8;
     for (int g = 0; g < ngroups; ++g) {
-      if (args->dtype == FLUXMI_BF16)
+      if (args->dtype != FLUXMI_FP8_E4M3)
         hipLaunchKernelGGL(grouped_gemm_generic_kernel<2>, dim3(grid), dim3(256), 0, s, p, g);
       else
         hipLaunchKernelGGL(grouped_gemm_generic_kernel<1>, dim3(grid), dim3(256), 0, s, p, g);
@@ -249,13 +253,15 @@ __global__ __launch_bounds__(256) void zero_f32x4_kernel(float4 *__restrict__ ds
     dst[i] = make_float4(0.f, 0.f, 0.f, 0.f);
 }
 
-__global__ __launch_bounds__(256) void cast_f32x4_bf16_kernel(const float4 *__restrict__ src, u32x2_t *__restrict__ dst,
+template <bool F16>
+__global__ __launch_bounds__(256) void cast_f32x4_half_kernel(const float4 *__restrict__ src, u32x2_t *__restrict__ dst,
                                                               int64_t nvec) {
+  auto cvt = [](float f) { return static_cast<uint32_t>(F16 ? float_to_f16_bits(f) : float_to_bf16_bits(f)); };
   for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < nvec; i += static_cast<int64_t>(gridDim.x) * 256) {
     const float4 v = src[i];
     u32x2_t o;
-    o[0] = static_cast<uint32_t>(float_to_bf16_bits(v.x)) | (static_cast<uint32_t>(float_to_bf16_bits(v.y)) << 16);
-    o[1] = static_cast<uint32_t>(float_to_bf16_bits(v.z)) | (static_cast<uint32_t>(float_to_bf16_bits(v.w)) << 16);
+    o[0] = cvt(v.x) | (cvt(v.y) << 16);
+    o[1] = cvt(v.z) | (cvt(v.w) << 16);
     __builtin_nontemporal_store(o, dst + i);
   }
 }
@@ -299,8 +305,12 @@ extern "C" int fluxmi_grouped_gemm_topk_reduce(const fluxmi_grouped_gemm_args *a
   const float *alpha = a.alpha;
   const int rc = run_grouped_gemm(&a, 1, &b, &d, &alpha, stream, false, ntokens);
   if (rc != FLUXMI_OK) return rc;
-  hipLaunchKernelGGL(cast_f32x4_bf16_kernel, dim3(grid), dim3(256), 0, s, static_cast<const float4 *>(workspace),
-                     static_cast<u32x2_t *>(out), nvec);
+  if (args->dtype == FLUXMI_FP16)
+    hipLaunchKernelGGL(cast_f32x4_half_kernel<true>, dim3(grid), dim3(256), 0, s, static_cast<const float4 *>(workspace),
+                       static_cast<u32x2_t *>(out), nvec);
+  else
+    hipLaunchKernelGGL(cast_f32x4_half_kernel<false>, dim3(grid), dim3(256), 0, s, static_cast<const float4 *>(workspace),
+                       static_cast<u32x2_t *>(out), nvec);
   FLUXMI_HIP_CHECK(hipGetLastError());
   return FLUXMI_OK;
 }

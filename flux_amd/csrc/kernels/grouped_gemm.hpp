@@ -90,11 +90,14 @@ struct GemmParams {
   const float *b_scale;
   int32_t a_scale_layout;  // FLUXMI_ASCALE_*
   int32_t b_scale_layout;  // FLUXMI_BSCALE_*
+  int32_t half_is_f16;     // 2-byte operands and outputs are fp16, not bf16 (read by the generic kernel; the MFMA
+                           // kernel is built once per 16-bit type)
 };
 
 
 // One launcher per element type, each in a translation unit of its own (the kernel is a long compile).
 int launch_grouped_gemm_bf16(const GemmParams &p, int grid, hipStream_t s);
+int launch_grouped_gemm_f16(const GemmParams &p, int grid, hipStream_t s);
 int launch_grouped_gemm_fp8(const GemmParams &p, int grid, hipStream_t s);
 int launch_grouped_gemm_fp8_blockscale(const GemmParams &p, int grid, hipStream_t s);
 

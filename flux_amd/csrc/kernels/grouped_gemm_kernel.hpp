@@ -19,10 +19,25 @@ __device__ __forceinline__ void load_to_lds16(const uint8_t *src, uint8_t *lds_b
   __builtin_amdgcn_global_load_lds((gbl_ptr_t)src, (lds_ptr_t)lds_base, 16, 0, 0);
 }
 
-// Two floats to packed bf16, round to nearest even (one v_cvt_pk_bf16_f32).
+// Which 16-bit float the 2-byte instantiation computes in: bf16 unless the including translation unit defines
+// FLUXMI_HALF_IS_F16 (the fp16 build of the same kernel: another MFMA opcode and another output cast, nothing else).
+#ifdef FLUXMI_HALF_IS_F16
+constexpr bool kHalfIsF16 = true;
+#else
+constexpr bool kHalfIsF16 = false;
+#endif
+
+// Two floats to the packed 16-bit output type (bf16: one v_cvt_pk_bf16_f32; fp16: two v_cvt_f16_f32 and a pack),
+// round to nearest even.  fp8 inputs always produce bf16.
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-  const f32x2 v = {lo, hi};
-  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+  if constexpr (kHalfIsF16) {
+    typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+    const f16x2 h = {static_cast<_Float16>(lo), static_cast<_Float16>(hi)};
+    return __builtin_bit_cast(uint32_t, h);
+  } else {
+    const f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+  }
 }
 
 // Source of the ring fills of a k-step past the end of K: every lane reads 16 zero bytes.
@@ -53,7 +68,10 @@ __device__ __forceinline__ void mfma_slot(int t, const i32x4 (&xf)[MBK][Geom<ELT
     // them at the loop's back edge.  Every accumulator is touched once per k-step, 63 MFMAs apart, and
     // the fragment operands come from LDS reads the compiler still tracks, so no hazard needs software
     // wait states here.
-    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(wf[j][0]), "v"(xf[i][0]));
+    if constexpr (kHalfIsF16)
+      asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(wf[j][0]), "v"(xf[i][0]));
+    else
+      asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(wf[j][0]), "v"(xf[i][0]));
   } else {
     i32x8 wa, xa;
 #pragma unroll
@@ -134,7 +152,6 @@ template <int ELT, int MB, int NB, bool FULL, bool OUT_F32, bool SCALED, bool SU
 __device__ __forceinline__ void store_tile(uint8_t *windows, const TileCtx &c, int g, int e, int row_base, int rows_e,
                                            int wrow0, int wcol0,
                                            const typename Geom<ELT>::Acc (&acc)[32 * MB / Geom<ELT>::BLK][32 * NB / Geom<ELT>::BLK]) {
-  static_assert(MB % 2 == 0, "a window holds 64 rows");
   constexpr int BLK = Geom<ELT>::BLK;
   constexpr int MBK = 32 * MB / BLK;
   constexpr int ELT_OUT = OUT_F32 ? 4 : 2;
@@ -161,7 +178,7 @@ __device__ __forceinline__ void store_tile(uint8_t *windows, const TileCtx &c, i
   const int d_rows = p->d_rows;
   const bool nt_stores = p->nt_stores != 0;  // wave-uniform
   const bool accumulate = !FULL && p->accumulate != 0;
-  if constexpr (ELT == 2 && !OUT_F32 && FULL && NB % 2 == 0) {
+  if constexpr (ELT == 2 && !OUT_F32 && FULL && NB % 2 == 0 && MB % 2 == 0) {
     // bf16 rows of whole tiles leave as whole 128-byte lines: two 32-column blocks per pass, packed to bf16
     // before the pass, so that the window (64 rows x 128 bytes) comes back as eight lanes x 16 bytes per row.
     // In 64-byte pieces a line is written in two halves at different times and part of the lines reach HBM
@@ -216,8 +233,9 @@ __device__ __forceinline__ void store_tile(uint8_t *windows, const TileCtx &c, i
   // 64-byte (bf16) / 128-byte (fp32) pieces: passes of 32 rows x 32 columns through the two 4 KiB halves of the
   // window in fp32, software-pipelined: while the rows of pass p come back from LDS and are stored, the
   // accumulators of pass p + 1 are already being written to the other half, so that the LDS round trip of a pass
-  // is not exposed.  Pass p = ((j * (MB / 2) + ip) * 2 + hh): column group j, 64-row group ip, its 32-row half hh.
-  constexpr int NPASS = NB * (MB / 2) * 2;
+  // is not exposed.  Pass p = j * MB + g: column group j, 32-row group g of the wave's rows; passes alternate between
+  // the two halves of the window.
+  constexpr int NPASS = NB * MB;
   float4 csj[NB];  // column scales of this lane's 4-column chunk in every column group
 #pragma unroll
   for (int j = 0; j < NB; ++j) {
@@ -228,11 +246,11 @@ __device__ __forceinline__ void store_tile(uint8_t *windows, const TileCtx &c, i
   // A lane holds one row of a block and groups of 4 consecutive columns of it: with 16x16 blocks one group,
   // columns 4 * (lane / 16); with 32x32 blocks four, columns 8q + 4 * (lane / 32).
   auto write_half = [&](auto PC) {
-    constexpr int ps = decltype(PC)::value, hh = ps & 1, blk = ps >> 1, ip = blk % (MB / 2), j = blk / (MB / 2);
+    constexpr int ps = decltype(PC)::value, hh = ps & 1, g32 = ps % MB, j = ps / MB;
     uint8_t *half = windows + hh * 4096;
 #pragma unroll
     for (int i2 = 0; i2 < 32 / BLK; ++i2) {
-      const int i = ip * (64 / BLK) + hh * (32 / BLK) + i2;
+      const int i = g32 * (32 / BLK) + i2;
       const int r = i2 * BLK + (lane & (BLK - 1));
 #pragma unroll
       for (int jj = 0; jj < 32 / BLK; ++jj) {
@@ -259,15 +277,15 @@ __device__ __forceinline__ void store_tile(uint8_t *windows, const TileCtx &c, i
     }
   };
   auto store_half = [&](auto PC, const float4 (&v)[4]) {
-    constexpr int ps = decltype(PC)::value, hh = ps & 1, blk = ps >> 1, ip = blk % (MB / 2), j = blk / (MB / 2);
+    constexpr int ps = decltype(PC)::value, g32 = ps % MB, j = ps / MB;
     const int col = wcol0 + j * 32 + cc * 4;
     const float4 cs = csj[j];
-    uint8_t *dp = dlane + (static_cast<int64_t>(ip) * 8 + hh * 4) * rowgroup_bytes + j * 32 * ELT_OUT;
+    uint8_t *dp = dlane + (static_cast<int64_t>(g32) * 4) * rowgroup_bytes + j * 32 * ELT_OUT;
 #pragma unroll
     for (int it = 0; it < 4; ++it, dp += rowgroup_bytes) {
       uint8_t *dst = dp;
       if constexpr (!FULL) {
-        const int m = wrow0 + ip * 64 + hh * 32 + it * 8 + rr0;
+        const int m = wrow0 + g32 * 32 + it * 8 + rr0;
         if (m >= rows_e || col >= n) continue;  // n % 4 == 0: a chunk is all in or all out
         if (scatter) {
           const int64_t drow = scatter[row_base + m];
@@ -278,14 +296,7 @@ __device__ __forceinline__ void store_tile(uint8_t *windows, const TileCtx &c, i
       float4 o = v[it];
       if constexpr (SCALED) o = make_float4(o.x * cs.x, o.y * cs.y, o.z * cs.z, o.w * cs.w);
       if constexpr (OUT_F32) {
-        if (accumulate) {
-          // Hardware fp32 atomic adds without return: sorted rows of one token meet in that token's row of D.
-          float *df = reinterpret_cast<float *>(dst);
-          unsafeAtomicAdd(df + 0, o.x);
-          unsafeAtomicAdd(df + 1, o.y);
-          unsafeAtomicAdd(df + 2, o.z);
-          unsafeAtomicAdd(df + 3, o.w);
-        } else if (nt_stores) {
+        if (nt_stores) {
           typedef float f32x4_t __attribute__((ext_vector_type(4)));
           const f32x4_t ov = {o.x, o.y, o.z, o.w};
           __builtin_nontemporal_store(ov, reinterpret_cast<f32x4_t *>(dst));
@@ -300,6 +311,54 @@ __device__ __forceinline__ void store_tile(uint8_t *windows, const TileCtx &c, i
       }
     }
   };
+  if constexpr (!FULL && OUT_F32) {
+    if (accumulate) {
+      // Top-k reduction in the epilogue: every result is added to row scatter[row] of the fp32 output with a hardware
+      // float atomic (no return value).  The block comes back from the window with 32 lanes per row, one float each,
+      // so that an atomic instruction covers two whole 128-byte lines (with the 8-lanes-per-row layout of the stores
+      // it would touch eight lines for 32 bytes each: four times the line operations at the L2 atomic units).
+      const int half_lane = lane >> 5, col_lane = lane & 31;
+      float csl[NB];
+#pragma unroll
+      for (int j = 0; j < NB; ++j) {
+        const int col = wcol0 + j * 32 + col_lane;
+        csl[j] = (col_scale && col < n) ? col_scale[static_cast<int64_t>(e) * n + col] : 1.f;
+      }
+      float *const df = reinterpret_cast<float *>(d);
+      auto read_rows = [&](auto PC, float (&f)[16]) {
+        constexpr int hh = decltype(PC)::value & 1;
+        const uint8_t *half = windows + hh * 4096;
+#pragma unroll
+        for (int it = 0; it < 16; ++it) {
+          const int rr = it * 2 + half_lane;
+          f[it] = *reinterpret_cast<const float *>(half + rr * 128 + (((col_lane >> 2) ^ ((rr >> 1) & 7)) << 4) + (col_lane & 3) * 4);
+        }
+      };
+      auto add_rows = [&](auto PC, const float (&f)[16]) {
+        constexpr int ps = decltype(PC)::value, g32 = ps % MB, j = ps / MB;
+        const int col = wcol0 + j * 32 + col_lane;
+#pragma unroll
+        for (int it = 0; it < 16; ++it) {
+          const int m = wrow0 + g32 * 32 + it * 2 + half_lane;
+          if (m >= rows_e || col >= n) continue;
+          const int64_t drow = scatter ? static_cast<int64_t>(scatter[row_base + m]) : static_cast<int64_t>(row_base + m);
+          if (drow < 0 || drow >= d_rows) continue;
+          unsafeAtomicAdd(df + drow * n + col, f[it] * csl[j]);
+        }
+      };
+      float fa[16], fb[16];
+      write_half(std::integral_constant<int, 0>{});
+      static_for<0, NPASS>([&](auto PC) {
+        constexpr int ps = decltype(PC)::value;
+        if constexpr ((ps & 1) == 0) read_rows(PC, fa);
+        else read_rows(PC, fb);
+        if constexpr (ps + 1 < NPASS) write_half(std::integral_constant<int, (ps + 1 < NPASS ? ps + 1 : 0)>{});
+        if constexpr ((ps & 1) == 0) add_rows(PC, fa);
+        else add_rows(PC, fb);
+      });
+      return;
+    }
+  }
   float4 va[4], vb[4];
   write_half(std::integral_constant<int, 0>{});
   static_for<0, NPASS>([&](auto PC) {
@@ -318,7 +377,8 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const uint8_t *base,
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(base), 0, static_cast<int>(n), 0x00020000);
 }
 // Where a work item lies.  kind: 0 a whole macro tile (4, 4); 1 the 128-row tile ending an expert (2, 4);
-// 2 a 256x128 piece (4, 2); 3 a 128x128 piece (2, 2); -1 an item without work; -2 past the last item.
+// 2 a 256x128 piece (4, 2); 3 a 128x128 piece (2, 2); 4 a 64x64 piece of an expert's last rows (1, 1); -1 an item
+// without work; -2 past the last item.
 // n0 is a column of the launch's virtual output: weight group g (a launch may multiply the same rows by up
 // to four weight tensors, each with an output of its own) occupies columns [g * npad, g * npad + n), npad =
 // n rounded up to whole macro tiles.
@@ -343,13 +403,18 @@ __device__ __forceinline__ int split_group(int &n0, int n, int ngroups) {
 // 128x128 pieces of a last round need 16 KiB per stage and have short k-steps (16 MFMAs per wave), so four
 // steps of look-ahead do not cover the memory latency: they run ten stages of 16 KiB, eight steps ahead.
 // Both stage counts divide ten, the number of k-steps over which the loop is unrolled.
+// The 64x64 pieces that the few last rows of an expert are cut into (one MFMA block row per wave and k-step) take
+// 8 KiB per stage: twenty stages, sixteen steps ahead, unrolled over twenty k-steps.
 template <int MB, int NB>
 struct Ring {
+  static_assert(MB != 1 || NB == 1, "64-row tiles exist as 64x64 pieces only");
+  static constexpr bool tiny = MB == 1;
   static constexpr bool deep = MB == 2 && NB == 2;
-  static constexpr int STG = deep ? 2 * STAGES : STAGES;
-  static constexpr int XB = deep ? X_TILE_BYTES / 2 : X_TILE_BYTES;  // X part of a stage
-  static constexpr int SB = deep ? STAGE_BYTES / 2 : STAGE_BYTES;    // a stage
-  static constexpr int LA = deep ? 8 : 4;                            // look-ahead in k-steps (even)
+  static constexpr int STG = tiny ? 4 * STAGES : (deep ? 2 * STAGES : STAGES);
+  static constexpr int XB = tiny ? X_TILE_BYTES / 4 : (deep ? X_TILE_BYTES / 2 : X_TILE_BYTES);  // X part of a stage
+  static constexpr int SB = tiny ? STAGE_BYTES / 4 : (deep ? STAGE_BYTES / 2 : STAGE_BYTES);     // a stage
+  static constexpr int LA = tiny ? 16 : (deep ? 8 : 4);                                          // look-ahead in k-steps (even)
+  static constexpr int TRIP = tiny ? 20 : 10;  // k-steps after which ring slot and fragment set repeat
 };
 
 // Operand addressing of a tile: buffer resources and this lane's byte offsets of its fill instructions.
@@ -725,25 +790,21 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
   FLUXMI_WAITCNT(63, 0);  // in registers before the first step's barrier lets anyone refill that slot
 
   // ---- main loop ----------------------------------------------------------------------------------
-  // Whole trips of ten k-steps while every k-step a trip requests (up to 9 + LA past its first one) is a whole
-  // one, then the remaining steps pair by pair with run-time ring slots.  An odd number of k-steps
+  // Whole trips of TRIP k-steps while every k-step a trip requests (up to TRIP - 1 + LA past its first one) is a
+  // whole one, then the remaining steps pair by pair with run-time ring slots.  An odd number of k-steps
   // ends with a phantom step on zero fragments.
-  const int nfast = nkf >= 10 + LA ? (nkf - (10 + LA)) / 10 + 1 : 0;  // trips with 10 * trip + 9 + LA < nkf
+  constexpr int TRIP = Ring<MB, NB>::TRIP;
+  const int nfast = nkf >= TRIP + LA ? (nkf - (TRIP + LA)) / TRIP + 1 : 0;  // trips with TRIP * trip + TRIP - 1 + LA < nkf
   int kbase = 0;  // byte offset along K of step 0 of the current trip
   for (int trip = 0; trip < nfast; ++trip) {
-    step(std::integral_constant<int, 0>{}, kbase, xa, wa, xb, wb);
-    step(std::integral_constant<int, 1>{}, kbase, xb, wb, xa, wa);
-    step(std::integral_constant<int, 2>{}, kbase, xa, wa, xb, wb);
-    step(std::integral_constant<int, 3>{}, kbase, xb, wb, xa, wa);
-    step(std::integral_constant<int, 4>{}, kbase, xa, wa, xb, wb);
-    step(std::integral_constant<int, 5>{}, kbase, xb, wb, xa, wa);
-    step(std::integral_constant<int, 6>{}, kbase, xa, wa, xb, wb);
-    step(std::integral_constant<int, 7>{}, kbase, xb, wb, xa, wa);
-    step(std::integral_constant<int, 8>{}, kbase, xa, wa, xb, wb);
-    step(std::integral_constant<int, 9>{}, kbase, xb, wb, xa, wa);
-    kbase += 10 * KBYTES;
+    static_for<0, TRIP / 2>([&](auto H) {
+      constexpr int u = 2 * decltype(H)::value;
+      step(std::integral_constant<int, u>{}, kbase, xa, wa, xb, wb);
+      step(std::integral_constant<int, u + 1>{}, kbase, xb, wb, xa, wa);
+    });
+    kbase += TRIP * KBYTES;
   }
-  for (int ks = 10 * nfast; ks < nk; ks += 2) {
+  for (int ks = TRIP * nfast; ks < nk; ks += 2) {
     step_dyn(ks, true, xa, wa, xb, wb);
     step_dyn(ks + 1, false, xb, wb, xa, wa);
   }
@@ -1108,10 +1169,14 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
   // Workgroups are dealt to XCDs round-robin; give each XCD a run of consecutive logical work items.
   const int virt = (grid % 8 == 0) ? (bid & 7) * (grid >> 3) + (bid >> 3) : bid;
 
-  // ---- total tile count (one wave-wide pass over splits) -> shape of the last round -----------------
-  int total_tiles = 0;
+  // ---- tile counts (one wave-wide pass over splits) -> shape of the last round ------------------------
+  // An expert whose last row tile holds 1 .. 64 rows is a candidate for a skinny tail: that row tile is then left
+  // out of the expert's ordinary tiles and computed after all of them as 64 x 64 pieces (below).
+  const bool cut_tail = (p.sched_flags & FLUXMI_SCHED_WHOLE_TAIL_TILES) == 0;
+  const bool half_tiles = (p.sched_flags & FLUXMI_SCHED_NO_HALF_TILES) == 0;
+  int total_tiles = 0, skinny_experts = 0;
   {
-    int row_carry = 0, acc_tiles = 0;
+    int row_carry = 0, acc_tiles = 0, acc_cand = 0;
     for (int e0 = 0; e0 < p.nexperts; e0 += 64) {
       const int ee = e0 + lane;
       int rows = ee < p.nexperts ? p.splits[ee] : 0;
@@ -1121,38 +1186,73 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
       if (begin > p.max_rows) begin = p.max_rows;
       if (end > p.max_rows) end = p.max_rows;
       int tiles = ((end - begin + BM - 1) / BM) * tiles_n;
+      int cand = (end > begin && ((end - begin - 1) & (BM - 1)) < 64) ? 1 : 0;
 #pragma unroll
-      for (int off = 32; off > 0; off >>= 1) tiles += __shfl_xor(tiles, off, 64);
+      for (int off = 32; off > 0; off >>= 1) {
+        tiles += __shfl_xor(tiles, off, 64);
+        cand += __shfl_xor(cand, off, 64);
+      }
       acc_tiles += tiles;
+      acc_cand += cand;
       row_carry += __shfl(incl, 63, 64);
     }
     total_tiles = __builtin_amdgcn_readfirstlane(acc_tiles);
+    skinny_experts = __builtin_amdgcn_readfirstlane(acc_cand);
   }
+  // Skinny tails.  A row tile with at most 64 rows costs a whole tile's weight traffic for a quarter of its MFMA
+  // work, and as an ordinary work item it occupies one compute unit for that long while the static schedule gives
+  // every unit the same number of items.  When such row tiles are few (their 64 x 64 pieces fill at most two
+  // rounds: long K, few column tiles) they are numbered after all ordinary tiles and cut along N into 64-column
+  // pieces, so that every unit streams an equal share of those experts' weights at the end; when they are many
+  // (short K, many column tiles) they already spread evenly as ordinary items and stay where they are.
+  const int skinny_tiles_all = skinny_experts * tiles_n;
+  const bool skinny_on = !BS && half_tiles && (p.sched_flags & FLUXMI_SCHED_NO_SKINNY_TAIL) == 0 && skinny_tiles_all > 0 &&
+                         ((p.sched_flags & FLUXMI_SCHED_FORCE_SKINNY_TAIL) != 0 || skinny_tiles_all * 4 <= 2 * grid);
+  const int skinny_items = skinny_on ? skinny_tiles_all * 4 : 0;
+  const int reg_tiles = total_tiles - (skinny_on ? skinny_tiles_all : 0);
   // Full rounds run whole macro tiles.  The tiles of the last, partly filled round are cut into
   // `pieces` parts (2 pieces of 256x128, or 4 of 128x128) when that still fits one round, so that the
   // chip does not idle while a fraction of the CUs finishes whole tiles.
   // Block-scaled launches run every tile as two 256 x 128 pieces (one column block of B's scales each).
-  const int full_items = BS ? 0 : (total_tiles / grid) * grid;
-  const int rem_tiles = total_tiles - full_items;
-  const bool cut_tail = (p.sched_flags & FLUXMI_SCHED_WHOLE_TAIL_TILES) == 0;
-  const bool half_tiles = (p.sched_flags & FLUXMI_SCHED_NO_HALF_TILES) == 0;
+  const int full_items = BS ? 0 : (reg_tiles / grid) * grid;
+  const int rem_tiles = reg_tiles - full_items;
   const int pieces = BS ? 2 : (!cut_tail ? 1 : (rem_tiles * 4 <= grid ? 4 : (rem_tiles * 2 <= grid ? 2 : 1)));
-  const int total_items = full_items + rem_tiles * pieces;
+  const int skinny_first = full_items + rem_tiles * pieces;  // first work item of the skinny pieces
+  const int total_items = skinny_first + skinny_items;
 
   // ---- schedule: walk the experts once, in step with this workgroup's increasing tile ids ----------
   // All of it is wave-uniform scalar work on the device-resident splits (no LDS, no host round trip).
+  // The walk is made twice: over the ordinary tiles, then (from work item skinny_first on) over the skinny pieces.
   int e = 0;
   int row_base = 0;   // sorted rows before expert e
-  int tile_base = 0;  // tiles before expert e
+  int tile_base = 0;  // ordinary tiles (second walk: skinny pieces) before expert e
   int rows_e = expert_rows(p, 0, 0);
-  int tiles_e = ((rows_e + BM - 1) / BM) * tiles_n;
+  bool in_skinny = false;
+  // Ordinary row tiles of an expert with `rows` rows / its skinny pieces.
+  auto is_skinny = [&](int rows) { return skinny_on && rows > 0 && ((rows - 1) & (BM - 1)) < 64; };
+  auto count_of = [&](int rows) {
+    const int mt = (rows + BM - 1) / BM;
+    if (in_skinny) return is_skinny(rows) ? tiles_n * 4 : 0;
+    return (mt - (is_skinny(rows) ? 1 : 0)) * tiles_n;
+  };
+  int tiles_e = count_of(rows_e);
 
   // Work item -> tile (items must be asked for in increasing order).
   auto locate = [&](int item) {
     TileDesc t = {-2, 0, 0, 0, 0, 0};
     if (item >= total_items) return t;
+    if (item >= skinny_first && !in_skinny) {  // restart the walk for the skinny pieces
+      in_skinny = true;
+      e = 0;
+      row_base = 0;
+      tile_base = 0;
+      rows_e = expert_rows(p, 0, 0);
+      tiles_e = count_of(rows_e);
+    }
     int tile = item, piece = 0;
-    if (item >= full_items) {
+    if (in_skinny) {
+      tile = item - skinny_first;
+    } else if (item >= full_items) {
       tile = full_items + (item - full_items) / pieces;
       piece = (item - full_items) % pieces;
     }
@@ -1162,15 +1262,29 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
       ++e;
       if (e < p.nexperts) {
         rows_e = expert_rows(p, e, row_base);
-        tiles_e = ((rows_e + BM - 1) / BM) * tiles_n;
+        tiles_e = count_of(rows_e);
       }
     }
     if (e >= p.nexperts) return t;
+    t.e = e;
+    t.row_base = row_base;
+    t.rows_e = rows_e;
+    if (in_skinny) {
+      // Piece `local` of the expert's last row tile: column tile local / 4 (over all weight groups), quarter local % 4.
+      const int local = tile - tile_base;
+      const int nt = local >> 2;
+      const int g = p.ngroups > 1 ? nt / tiles_n1 : 0;
+      t.m0 = ((rows_e - 1) / BM) * BM;
+      t.n0 = (nt - g * tiles_n1) * BN + (local & 3) * 64;
+      t.kind = t.n0 < p.n ? 4 : -1;
+      t.n0 += g * tiles_n1 * BN;
+      return t;
+    }
     // Order inside an expert: row tiles are cut into groups of at most p.raster_rows (8 unless tuned); a group is walked
     // column-major over all weight panels before the next group starts.  32 consecutive tiles (one
     // XCD's share of a round) then cover about 8 row tiles x 4 panels: 12 distinct operand tiles per
     // k-step for 32 CUs.
-    const int m_tiles = (rows_e + BM - 1) / BM;
+    const int m_tiles = (rows_e + BM - 1) / BM - (is_skinny(rows_e) ? 1 : 0);
     const int ngroups_m = (m_tiles + p.raster_rows - 1) / p.raster_rows;
     const int gm = (m_tiles + ngroups_m - 1) / ngroups_m;  // group height, <= raster_rows
     const int local = tile - tile_base;
@@ -1180,9 +1294,6 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
     const int in_group = local - group * gm * tiles_n;
     const int nt = in_group / group_rows;
     const int mt = group_first + (in_group - nt * group_rows);
-    t.e = e;
-    t.row_base = row_base;
-    t.rows_e = rows_e;
     t.m0 = mt * BM;
     const int g = p.ngroups > 1 ? nt / tiles_n1 : 0;
     const int gcol = g * tiles_n1 * BN;  // first virtual column of the weight group
@@ -1219,6 +1330,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
       else if (cur.kind == 1) gemm_tile<ELT, 2, 4>(p, smem, c, cur, next, pf);
       else if (cur.kind == 2) gemm_tile<ELT, 4, 2>(p, smem, c, cur, next, pf);
       else if (cur.kind == 3) gemm_tile<ELT, 2, 2>(p, smem, c, cur, next, pf);
+      else if (cur.kind == 4) gemm_tile<ELT, 1, 1>(p, smem, c, cur, next, pf);
     }
     cur = next;
   }

@@ -141,7 +141,7 @@ __global__ __launch_bounds__(kThreads) void route_scatter_kernel(
     const int32_t *__restrict__ splits_ws, int32_t *__restrict__ splits_out, int32_t *__restrict__ offsets_out,
     int32_t *__restrict__ scatter_index, int32_t *__restrict__ gather_index,
     int32_t *__restrict__ topk_index) {
-  extern __shared__ int32_t s_mem[];  // [nexperts] offsets, [kWavesPerBlock][nexperts] running, FUSED: [nexperts] totals
+  extern __shared__ int32_t s_mem[];  // [nexperts] offsets, [kWavesPerBlock][nexperts] running, FUSED: [2][nexperts] totals, sums ahead
   int32_t *s_off = s_mem;
   const int wave = threadIdx.x >> 6;
   const int lane = threadIdx.x & 63;
@@ -150,18 +150,43 @@ __global__ __launch_bounds__(kThreads) void route_scatter_kernel(
   const int chunk0 = blockIdx.x * kWavesPerBlock;
 
   if constexpr (FUSED_SCAN) {
+    // Column sums of the chunks x experts table, per expert: over the chunks ahead of this workgroup's four (s_before)
+    // and over all chunks (s_tot).  All lanes sweep the table in its memory order (coalesced, independent loads, four
+    // in flight per lane) and add into LDS; the table is small (C4: 192 x 64) and sits in L2.
+    int32_t *s_before = s_tot + nexperts;
     for (int e = threadIdx.x; e < nexperts; e += kThreads) {
-      int sum = 0;
-      int c = 0;
-      for (; c < chunk0 && c < nchunks; ++c) sum += base[static_cast<size_t>(c) * nexperts + e];
+      s_tot[e] = 0;
+      s_before[e] = 0;
+    }
+    __syncthreads();
+    const int total = nchunks * nexperts;
+    const int before_end = (chunk0 < nchunks ? chunk0 : nchunks) * nexperts;
+    for (int f0 = threadIdx.x; f0 < total; f0 += 4 * kThreads) {
+      int32_t v[4];
 #pragma unroll
-      for (int w = 0; w < kWavesPerBlock; ++w, ++c) {
-        s_mem[nexperts + w * nexperts + e] = sum;  // rows of expert e in the chunks ahead of chunk0 + w
-        if (c < nchunks) sum += base[static_cast<size_t>(c) * nexperts + e];
+      for (int u = 0; u < 4; ++u) {
+        const int f = f0 + u * kThreads;
+        v[u] = f < total ? base[f] : 0;
       }
-      for (; c < nchunks; ++c) sum += base[static_cast<size_t>(c) * nexperts + e];
-      s_tot[e] = sum;
-      if (blockIdx.x == 0 && splits_out) splits_out[e] = sum;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int f = f0 + u * kThreads;
+        if (v[u] != 0) {
+          const int e = f % nexperts;
+          atomicAdd(&s_tot[e], v[u]);
+          if (f < before_end) atomicAdd(&s_before[e], v[u]);
+        }
+      }
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < nexperts; e += kThreads) {
+      int sum = s_before[e];
+#pragma unroll
+      for (int w = 0; w < kWavesPerBlock; ++w) {
+        s_mem[nexperts + w * nexperts + e] = sum;  // rows of expert e in the chunks ahead of chunk0 + w
+        if (chunk0 + w < nchunks) sum += base[static_cast<size_t>(chunk0 + w) * nexperts + e];
+      }
+      if (blockIdx.x == 0 && splits_out) splits_out[e] = s_tot[e];
     }
     __syncthreads();
   }
@@ -327,7 +352,7 @@ int route_sort_on_workspace(const int32_t *choosed, int32_t ntokens, int32_t top
     // Two launches: every scatter workgroup scans the histogram table itself.  With no pairs one block still
     // runs to publish splits and offsets (all zero).
     hipLaunchKernelGGL(route_scatter_kernel<true>, dim3(nblocks > 0 ? nblocks : 1), dim3(kThreads),
-                       (2 + kWavesPerBlock) * nexperts * sizeof(int32_t), s, choosed, npairs, topk, nexperts, nchunks,
+                       (3 + kWavesPerBlock) * nexperts * sizeof(int32_t), s, choosed, npairs, topk, nexperts, nchunks,
                        idbits, hist, splits_ws, splits, offsets, scatter_index, gather_index, topk_index);
   } else {
     hipLaunchKernelGGL(route_scan_kernel, dim3((nexperts + kWavesPerBlock - 1) / kWavesPerBlock),

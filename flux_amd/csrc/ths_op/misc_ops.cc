@@ -289,7 +289,7 @@ torch::Tensor topk_weighted_gather_reduce(std::vector<torch::Tensor> inputs, tor
                                           std::optional<torch::Tensor> row_weight, double scale) {
   TORCH_CHECK(!inputs.empty(), "inputs must not be empty");
   const at::ScalarType st = inputs[0].scalar_type();
-  TORCH_CHECK(st == at::kBFloat16 || st == at::kFloat, "inputs must be bfloat16 or float32");
+  TORCH_CHECK(st == at::kBFloat16 || st == at::kFloat || st == at::kHalf, "inputs must be bfloat16, float16 or float32");
   const int64_t m = inputs[0].size(0), n = inputs[0].size(1);
   TORCH_CHECK(topk >= 1 && m % topk == 0, "rows ", m, " not a multiple of topk ", topk);
   FLUX_AMD_CHECK_INPUT(routing_idx, at::kInt);
@@ -306,8 +306,8 @@ torch::Tensor topk_weighted_gather_reduce(std::vector<torch::Tensor> inputs, tor
     TORCH_CHECK(row_weight->numel() == m, "row_weight must be [M]");
     w = row_weight->data_ptr<float>();
   }
-  torch::Tensor out = torch::empty({m / topk, n}, inputs[0].options().dtype(at::kBFloat16));
-  check_status(fluxmi_topk_gather_reduce(ptrs.data(), static_cast<int32_t>(ptrs.size()), st == at::kFloat ? 1 : 0,
+  torch::Tensor out = torch::empty({m / topk, n}, inputs[0].options().dtype(st == at::kHalf ? at::kHalf : at::kBFloat16));
+  check_status(fluxmi_topk_gather_reduce(ptrs.data(), static_cast<int32_t>(ptrs.size()), st == at::kFloat ? 1 : (st == at::kHalf ? 2 : 0),
                                          routing_idx.data_ptr<int32_t>(), w, static_cast<float>(scale),
                                          static_cast<int32_t>(m / topk), static_cast<int32_t>(topk),
                                          static_cast<int32_t>(n), out.data_ptr(), current_stream()),

@@ -17,6 +17,13 @@ namespace flux_amd {
 namespace {
 // Schedule forced on every launch of this thread while a profiler tries it.
 thread_local const GemmLaunchTuning *t_tuning_override = nullptr;
+// Form of layer1's reduction forced on this thread while a profiler tries it: 0 none, 1 fused, 2 two-pass.
+thread_local int t_reduce_override = 0;
+
+struct ScopedReduceOverride {
+  explicit ScopedReduceOverride(int form) { t_reduce_override = form; }
+  ~ScopedReduceOverride() { t_reduce_override = 0; }
+};
 
 struct ScopedTuningOverride {
   explicit ScopedTuningOverride(const GemmLaunchTuning *t) { t_tuning_override = t; }
@@ -43,25 +50,22 @@ GemmShapeKey shape_key(const fluxmi_grouped_gemm_args &args, int32_t ngroups) {
 // Times `run` (one whole forward) under every candidate schedule on the current stream, 5 warm-up and 10
 // timed calls each like the reference's profiling loops (gemm_grouped_v3_ag_scatter.cc:540-590), records
 // them in `ctx` and registers the fastest for `key`.
+// Mean time in ms of one call of `run` on the current stream: 5 warm-up and 10 timed calls.
 template <class F>
-void profile_schedules(const GemmShapeKey &key, ProfilingContext *ctx, F &&run) {
+float time_calls(F &&run) {
   constexpr int kWarmIters = 5, kIters = 10;
   hipStream_t stream = static_cast<hipStream_t>(current_stream());
   hipEvent_t e0, e1;
   FLUX_AMD_HIP_CHECK(hipEventCreate(&e0));
   FLUX_AMD_HIP_CHECK(hipEventCreate(&e1));
+  float ms = 0.f;
   try {
-    for (const GemmLaunchTuning &cand : gemm_tuning_candidates()) {
-      ScopedTuningOverride scope(&cand);
-      for (int i = 0; i < kWarmIters; ++i) run();
-      FLUX_AMD_HIP_CHECK(hipEventRecord(e0, stream));
-      for (int i = 0; i < kIters; ++i) run();
-      FLUX_AMD_HIP_CHECK(hipEventRecord(e1, stream));
-      FLUX_AMD_HIP_CHECK(hipEventSynchronize(e1));
-      float ms = 0.f;
-      FLUX_AMD_HIP_CHECK(hipEventElapsedTime(&ms, e0, e1));
-      ctx->add(key, cand, ms / kIters);
-    }
+    for (int i = 0; i < kWarmIters; ++i) run();
+    FLUX_AMD_HIP_CHECK(hipEventRecord(e0, stream));
+    for (int i = 0; i < kIters; ++i) run();
+    FLUX_AMD_HIP_CHECK(hipEventRecord(e1, stream));
+    FLUX_AMD_HIP_CHECK(hipEventSynchronize(e1));
+    FLUX_AMD_HIP_CHECK(hipEventElapsedTime(&ms, e0, e1));
   } catch (...) {
     (void)hipEventDestroy(e0);
     (void)hipEventDestroy(e1);
@@ -69,6 +73,15 @@ void profile_schedules(const GemmShapeKey &key, ProfilingContext *ctx, F &&run) 
   }
   FLUX_AMD_HIP_CHECK(hipEventDestroy(e0));
   FLUX_AMD_HIP_CHECK(hipEventDestroy(e1));
+  return ms / kIters;
+}
+
+template <class F>
+void profile_schedules(const GemmShapeKey &key, ProfilingContext *ctx, F &&run) {
+  for (const GemmLaunchTuning &cand : gemm_tuning_candidates()) {
+    ScopedTuningOverride scope(&cand);
+    ctx->add(key, cand, time_calls(run));
+  }
   TuningTable::instance().add(key, ctx->record_best(key));
 }
 }  // namespace
@@ -121,8 +134,9 @@ GemmGroupedV3AGScatter::GemmGroupedV3AGScatter(DistEnvTPWithEP tp_env, MoeArgume
                   moe_args.nexperts > 0 && moe_args.topk > 0,
               "MoeArguments sizes must be positive");
   to_fluxmi_dtype(moe_args.input_dtype);
-  TORCH_CHECK(moe_args.output_dtype == at::ScalarType::BFloat16,
-              "output dtype must be bfloat16 (fp8 inputs produce bf16 too), got ", moe_args.output_dtype);
+  TORCH_CHECK(moe_args.output_dtype == moe_output_dtype(moe_args.input_dtype),
+              "output dtype must be ", moe_output_dtype(moe_args.input_dtype), " for ", moe_args.input_dtype,
+              " inputs (fp16 gives fp16; bf16 and fp8 give bf16), got ", moe_args.output_dtype);
   // Persistent scratch sized from the constructor arguments, like the reference's input_buffer
   // (gemm_grouped_v3_ag_scatter.cc:86-101): the inverse permutation of scatter_index.
   gather_index_ = torch::empty({static_cast<int64_t>(moe_args.max_ntokens) * moe_args.topk},
@@ -301,7 +315,7 @@ void GemmGroupedV3GatherRS::lazy_init(const torch::Tensor &like) {
   // that the layer has a single rounding.  FLUX_AMD_INTER_DTYPE=bf16 restores the reference's data flow.
   // Zero-filled once, as the reference does (init_buffer: torch::zeros): rows the GEMM never writes
   // (sum(splits) < M) then read as zeros in the reduce instead of stale memory.
-  auto opts = like.options().dtype(inter_fp32_ ? at::kFloat : at::kBFloat16);
+  auto opts = like.options().dtype(inter_fp32_ ? at::kFloat : moe_output_dtype(like.scalar_type()));
   for (int64_t g = 0; g < max_input_groups_; ++g) inter_.push_back(torch::zeros({max_m_, n_dim_}, opts));
   splits_dev_ = torch::empty({num_experts_}, like.options().dtype(at::kInt));
   token_of_row_ = torch::empty({max_m_}, like.options().dtype(at::kInt));
@@ -348,13 +362,31 @@ torch::Tensor GemmGroupedV3GatherRS::forward_impl(
 
   lazy_init(inputs[0]);
   const int64_t ntokens = global_m / topk_;
-  torch::Tensor out = torch::empty({ntokens, n_dim_}, inputs[0].options().dtype(at::kBFloat16));
+  const bool f16 = st == at::ScalarType::Half;
+  torch::Tensor out = torch::empty({ntokens, n_dim_}, inputs[0].options().dtype(moe_output_dtype(st)));
   if (global_m == 0) return out;
   splits_dev_.copy_(splits_cpu.contiguous(), /*non_blocking=*/true);
 
-  // One input group, an fp32 scratch at hand and the fused form asked for: the reduction runs in the GEMM's
-  // epilogue.  (By shape nothing selects it yet: the two-pass form is the default everywhere.)
-  const bool fused = fused_mode_ == 1 && groups == 1 && inter_fp32_;
+  // One input group and an fp32 scratch at hand: the reduction may run in the GEMM's epilogue.  It does when
+  // FLUX_AMD_LAYER1_REDUCE=fused asks for it, or when profiling() found it faster for this shape (a tuning record
+  // with reduce=fused); FLUX_AMD_LAYER1_REDUCE=twopass overrides the table.  Without either the two-pass form runs:
+  // it is the faster one on every shape measured so far and deterministic for every top-k.
+  bool want_fused = fused_mode_ == 1;
+  if (fused_mode_ == 0) {
+    if (t_reduce_override != 0) {
+      want_fused = t_reduce_override == 1;
+    } else {
+      GemmShapeKey key;
+      key.dtype = to_fluxmi_dtype(st);
+      key.nexperts = static_cast<int32_t>(num_experts_);
+      key.n = static_cast<int32_t>(n_dim_);
+      key.k = static_cast<int32_t>(k);
+      key.max_rows = static_cast<int32_t>(m);
+      key.ngroups = 1;
+      if (auto t = TuningTable::instance().find(key)) want_fused = t->reduce_fused != 0;
+    }
+  }
+  const bool fused = want_fused && groups == 1 && inter_fp32_;
   std::vector<const void *> group_ptrs;
   for (size_t g = 0; g < groups; ++g) {
     const float *alpha = nullptr, *row = nullptr, *col = nullptr, *scalar = nullptr;
@@ -408,7 +440,7 @@ torch::Tensor GemmGroupedV3GatherRS::forward_impl(
     run_grouped_gemm(inputs[g], weights[g], splits_dev_, inter_[g], nullptr, m, alpha, row, col, scalar, sm_margin);
     group_ptrs.push_back(inter_[g].data_ptr());
   }
-  check_status(fluxmi_topk_gather_reduce(group_ptrs.data(), static_cast<int32_t>(groups), inter_fp32_ ? 1 : 0,
+  check_status(fluxmi_topk_gather_reduce(group_ptrs.data(), static_cast<int32_t>(groups), (inter_fp32_ ? 1 : 0) | (f16 ? 2 : 0),
                                          routing_idx.data_ptr<int32_t>(), nullptr, 1.0f,
                                          static_cast<int32_t>(ntokens), static_cast<int32_t>(topk_),
                                          static_cast<int32_t>(n_dim_), out.data_ptr(), current_stream()),
@@ -450,7 +482,26 @@ torch::Tensor GemmGroupedV3GatherRS::profiling(
   key.k = static_cast<int32_t>(input.size(1));
   key.max_rows = static_cast<int32_t>(input.size(0));
   key.ngroups = 1;
-  if (key.max_rows > 0) profile_schedules(key, ctx, run);
+  if (key.max_rows > 0) {
+    {
+      ScopedReduceOverride twopass(fused_mode_ == 0 ? 2 : 0);  // an earlier record must not switch forms mid-sweep
+      profile_schedules(key, ctx, run);
+    }
+    // With the fastest schedule registered: the other form of the reduction (atomic adds in the GEMM's epilogue
+    // instead of GEMM + gather-reduce kernel), when this op could run either.  Its time ranks among the two-pass
+    // timings of every schedule; the fastest entry becomes the record.
+    if (fused_mode_ == 0 && inter_fp32_) {
+      GemmLaunchTuning best = *TuningTable::instance().find(key);
+      best.reduce_fused = 1;
+      float ms = 0.f;
+      {
+        ScopedReduceOverride fused(1);
+        ms = time_calls(run);
+      }
+      ctx->add(key, best, ms);
+      TuningTable::instance().add(key, ctx->record_best(key));
+    }
+  }
   return run();  // with the schedule just registered
 }
 
@@ -484,7 +535,7 @@ torch::Tensor GemmGroupedV3::forward(torch::Tensor input, torch::Tensor splits_c
   TORCH_CHECK(weight_.size(2) == input.size(1), "weight 2-dim mismatch: ", weight_.size(2), " != ", input.size(1));
   TORCH_CHECK(splits_cpu.size(0) == weight_.size(0), "splits 0-dim mismatch: ", splits_cpu.size(0), " != ",
               weight_.size(0));
-  torch::Tensor out = torch::empty({input.size(0), weight_.size(1)}, input.options().dtype(at::kBFloat16));
+  torch::Tensor out = torch::empty({input.size(0), weight_.size(1)}, input.options().dtype(moe_output_dtype(input.scalar_type())));
   if (input.size(0) == 0) return out;
   torch::Tensor splits_dev = splits_cpu.to(at::kInt).to(input.device(), /*non_blocking=*/true);
   run_grouped_gemm(input, weight_, splits_dev, out, nullptr, input.size(0), nullptr, nullptr, nullptr, nullptr, 0);

@@ -62,7 +62,8 @@ PYBIND11_MODULE(flux_ths_pybind, m) {
       .def("__repr__", &TuningRecord::to_string)
       .def_property_readonly("shape", [](const TuningRecord &r) { return r.key.to_string(); })
       .def_property_readonly("raster_rows", [](const TuningRecord &r) { return r.best.raster_rows; })
-      .def_property_readonly("sched_flags", [](const TuningRecord &r) { return r.best.sched_flags; });
+      .def_property_readonly("sched_flags", [](const TuningRecord &r) { return r.best.sched_flags; })
+      .def_property_readonly("reduce_fused", [](const TuningRecord &r) { return r.best.reduce_fused != 0; });
 
   py::class_<GemmGroupedV3AGScatter>(m, "GemmGroupedV3AGScatter")
       .def(py::init<DistEnvTPWithEP, MoeArguments>(), py::arg("tp_env"), py::arg("moe_args"))

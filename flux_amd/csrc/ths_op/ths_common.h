@@ -29,8 +29,15 @@ inline bool is_fp8(at::ScalarType t) { return t == at::ScalarType::Float8_e4m3fn
 inline int32_t to_fluxmi_dtype(at::ScalarType t) {
   if (t == at::ScalarType::BFloat16) return FLUXMI_BF16;
   if (t == at::ScalarType::Float8_e4m3fn) return FLUXMI_FP8_E4M3;
-  TORCH_CHECK(false, "flux_amd: unsupported dtype ", t, " (bf16 and float8_e4m3fn are built)");
+  if (t == at::ScalarType::Half) return FLUXMI_FP16;
+  TORCH_CHECK(false, "flux_amd: unsupported dtype ", t, " (bf16, fp16 and float8_e4m3fn are built)");
   return -1;
+}
+
+// Output dtype of the two MoE ops for an operand dtype: fp16 in gives fp16 out, bf16 and fp8 in give bf16 out
+// (test/python/moe_ag_scatter/test_moe_ag.py:424-430 OUT_DTYPE_MAP; gemm_grouped_v3_gather_rs.cc:53-63).
+inline at::ScalarType moe_output_dtype(at::ScalarType in) {
+  return in == at::ScalarType::Half ? at::ScalarType::Half : at::ScalarType::BFloat16;
 }
 
 #define FLUX_AMD_CHECK_INPUT(x, st)                                                        \

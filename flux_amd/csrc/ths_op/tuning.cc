@@ -14,7 +14,7 @@ namespace flux_amd {
 
 std::string GemmShapeKey::to_string() const {
   std::ostringstream ss;
-  ss << "dtype=" << (dtype == FLUXMI_BF16 ? "bf16" : "e4m3") << " experts=" << nexperts << " n=" << n << " k=" << k
+  ss << "dtype=" << (dtype == FLUXMI_BF16 ? "bf16" : (dtype == FLUXMI_FP16 ? "f16" : "e4m3")) << " experts=" << nexperts << " n=" << n << " k=" << k
      << " rows=" << max_rows << " groups=" << ngroups;
   return ss.str();
 }
@@ -22,6 +22,7 @@ std::string GemmShapeKey::to_string() const {
 std::string GemmLaunchTuning::to_string() const {
   std::ostringstream ss;
   ss << "raster_rows=" << raster_rows << " sched_flags=" << sched_flags;
+  if (reduce_fused) ss << " reduce=fused";
   return ss.str();
 }
 
@@ -32,6 +33,9 @@ std::vector<GemmLaunchTuning> gemm_tuning_candidates() {
   for (int32_t flags : {0, FLUXMI_SCHED_WHOLE_TAIL_TILES, FLUXMI_SCHED_NO_HALF_TILES,
                         FLUXMI_SCHED_WHOLE_TAIL_TILES | FLUXMI_SCHED_NO_HALF_TILES})
     for (int32_t rows : {8, 4, 16}) out.push_back(GemmLaunchTuning{rows, flags});
+  // where the few last rows of an expert run: as 64 x 64 pieces behind all other tiles, or in place
+  out.push_back(GemmLaunchTuning{8, FLUXMI_SCHED_NO_SKINNY_TAIL});
+  out.push_back(GemmLaunchTuning{8, FLUXMI_SCHED_FORCE_SKINNY_TAIL});
   return out;
 }
 
@@ -99,8 +103,15 @@ size_t TuningTable::load_text(const std::string &text) {
       if (name == "dtype") {
         if (value == "bf16") key.dtype = FLUXMI_BF16;
         else if (value == "e4m3") key.dtype = FLUXMI_FP8_E4M3;
+        else if (value == "f16") key.dtype = FLUXMI_FP16;
         else fail("unknown dtype '" + value + "'");
         seen |= 1;
+        continue;
+      }
+      if (name == "reduce") {  // optional: the form of layer1's top-k reduction
+        if (value == "fused") t.reduce_fused = 1;
+        else if (value == "twopass") t.reduce_fused = 0;
+        else fail("unknown reduce form '" + value + "'");
         continue;
       }
       char *end = nullptr;
@@ -116,7 +127,8 @@ size_t TuningTable::load_text(const std::string &text) {
       else fail("unknown field '" + name + "'");
     }
     if (seen != 255) fail("missing fields");
-    if (t.raster_rows > 1024 || (t.sched_flags & ~(FLUXMI_SCHED_WHOLE_TAIL_TILES | FLUXMI_SCHED_NO_HALF_TILES)))
+    if (t.raster_rows > 1024 || (t.sched_flags & ~(FLUXMI_SCHED_WHOLE_TAIL_TILES | FLUXMI_SCHED_NO_HALF_TILES | FLUXMI_SCHED_NO_SKINNY_TAIL |
+                                                  FLUXMI_SCHED_FORCE_SKINNY_TAIL)))
       fail("raster_rows / sched_flags out of range");
     add(key, t);
     ++count;

@@ -29,7 +29,10 @@ struct GemmShapeKey {
 struct GemmLaunchTuning {
   int32_t raster_rows = 0;  // 0 = the kernel's default
   int32_t sched_flags = 0;  // FLUXMI_SCHED_*
-  bool operator==(const GemmLaunchTuning &o) const { return raster_rows == o.raster_rows && sched_flags == o.sched_flags; }
+  int32_t reduce_fused = 0;  // layer1 only: 1 = the top-k reduction runs in the GEMM's epilogue, 0 = GEMM, then gather-reduce
+  bool operator==(const GemmLaunchTuning &o) const {
+    return raster_rows == o.raster_rows && sched_flags == o.sched_flags && reduce_fused == o.reduce_fused;
+  }
   std::string to_string() const;
 };
 

@@ -28,8 +28,10 @@ typedef enum fluxmi_status {
 } fluxmi_status;
 
 typedef enum fluxmi_dtype {
-  FLUXMI_BF16 = 0,    /* bfloat16 operands, fp32 accumulate */
-  FLUXMI_FP8_E4M3 = 1 /* OCP e4m3 (torch.float8_e4m3fn) operands, fp32 accumulate */
+  FLUXMI_BF16 = 0,     /* bfloat16 operands, fp32 accumulate, bf16 (or fp32) output */
+  FLUXMI_FP8_E4M3 = 1, /* OCP e4m3 (torch.float8_e4m3fn) operands, fp32 accumulate, bf16 (or fp32) output */
+  FLUXMI_FP16 = 2      /* IEEE half operands, fp32 accumulate, fp16 (or fp32) output: the reference's fp16 variants of
+                          both MoE ops (src/generator/gen_moe_ag_scatter.cc:26-39, gen_moe_gather_rs.cc:25-45) */
 } fluxmi_dtype;
 
 /* Library version (major*10000 + minor*100 + patch) and the last error text of the calling thread. */
@@ -99,14 +101,15 @@ int fluxmi_moe_gather_index(const int32_t *scatter_index, int32_t nrows, int32_t
  *         bf16( acc[n] * (alpha ? alpha[e] : 1) * (row_scale ? row_scale[r] : 1)
  *                      * (col_scale ? col_scale[e*N + n] : 1) * scalar_scale )
  *
- * A is row-major [*, K] (lda = K), B is [E, N, K] with K contiguous, D is row-major [*, N] bf16.
+ * A is row-major [*, K] (lda = K), B is [E, N, K] with K contiguous, D is row-major [*, N] in the 16-bit output
+ * type of `dtype` (bf16 for bf16 and fp8 operands, fp16 for fp16 operands; "bf16" below stands for that type).
  * `splits` is a DEVICE int32 array of `nexperts` row counts; the tile schedule is derived from it on
  * the device, so the host never reads it.  `max_rows` is an upper bound of sum(splits) (ntokens*topk);
  * rows beyond sum(splits) are not touched.
  *
  * Limits: 1 <= nexperts <= 1024 (FLUXMI_ERR_UNSUPPORTED beyond).  Two kernels stand behind the call.  The
  * MFMA kernel takes every shape with
- *   - rows of K a multiple of 16 bytes: K % 8 == 0 (bf16), K % 16 == 0 (fp8); a last partial 64-byte step of
+ *   - rows of K a multiple of 16 bytes: K % 8 == 0 (bf16, fp16), K % 16 == 0 (fp8); a last partial 64-byte step of
  *     K is padded with zeros inside the kernel at full speed;
  *   - N % 4 == 0; a, b 16-byte aligned; d 8-byte (bf16) / 16-byte (fp32) aligned; col_scale 16-byte aligned;
  *   - one expert's weights below 4 GiB (N * K * element size), and with `gather_a`: a_rows > 0 and the whole
@@ -131,7 +134,7 @@ typedef struct fluxmi_grouped_gemm_args {
   const float *row_scale;   /* device [max_rows] or NULL, indexed by sorted row */
   const float *col_scale;   /* device [E, N] or NULL */
   float scalar_scale;       /* host scalar, 1.0f for none (Flux `input_scale[0]` is passed by pointer below) */
-  int32_t d_fp32;           /* 0: D is bf16; 1: D is fp32 [max_rows, N] (unrounded layer1 intermediate) */
+  int32_t d_fp32;           /* 0: D is bf16 (fp16 for FLUXMI_FP16); 1: D is fp32 [max_rows, N] (unrounded layer1 intermediate) */
   const float *scalar_scale_dev; /* device [1] or NULL; multiplied in if given */
   /* Launch tuning; all zero = defaults.  None of them changes a result bit. */
   int32_t cu_margin;     /* compute units left free for other work (Flux `sm_margin`) */
@@ -142,6 +145,8 @@ typedef struct fluxmi_grouped_gemm_args {
 
 #define FLUXMI_SCHED_WHOLE_TAIL_TILES 1 /* do not cut the tiles of the last, partly filled round into pieces */
 #define FLUXMI_SCHED_NO_HALF_TILES 2    /* run the last row tile of an expert 256 rows high even if 128 cover it, and the last column tile 256 wide even if 128 cover it */
+#define FLUXMI_SCHED_NO_SKINNY_TAIL 4    /* never move the last row tiles of experts that hold at most 64 rows behind all other tiles as 64 x 64 pieces */
+#define FLUXMI_SCHED_FORCE_SKINNY_TAIL 8 /* always do so (by default only when those pieces fill at most two rounds of the launch) */
 
 size_t fluxmi_grouped_gemm_workspace_bytes(const fluxmi_grouped_gemm_args *args);
 int fluxmi_grouped_gemm(const fluxmi_grouped_gemm_args *args, void *workspace,
@@ -227,13 +232,14 @@ int fluxmi_grouped_gemm_multi(const fluxmi_grouped_gemm_args *args, int32_t ngro
  *                       w[r] * float(in[g][r, n]) ),   r = routing_idx[t*topk + j],
  *   w[r] = row_weight ? row_weight[r] : 1;  fp32 accumulation in the order g-major then j; one rounding at
  *   the end.
- * `in` is an array (on the HOST) of `ngroups` device pointers to row-major [ntokens*topk, n] matrices, bf16,
- * or fp32 when `in_fp32` != 0 (the unrounded intermediate of fluxmi_grouped_gemm with d_fp32 = 1).  Entries of
+ * `in` is an array (on the HOST) of `ngroups` device pointers to row-major [ntokens*topk, n] matrices.
+ * `io_format` names the element types: 0 bf16 in, bf16 out; 1 fp32 in (the unrounded intermediate of
+ * fluxmi_grouped_gemm with d_fp32 = 1), bf16 out; 2 fp16 in, fp16 out; 3 fp32 in, fp16 out.  Entries of
  * routing_idx outside [0, ntokens*topk) name no row: they are skipped (negative = a dropped pair) and never
  * dereferenced.
  * Requirements: n % 8 == 0, 1 <= ngroups <= 4, 1 <= topk <= 64.
  * ---------------------------------------------------------------------------------------------- */
-int fluxmi_topk_gather_reduce(const void *const *in, int32_t ngroups, int32_t in_fp32,
+int fluxmi_topk_gather_reduce(const void *const *in, int32_t ngroups, int32_t io_format,
                               const int32_t *routing_idx, const float *row_weight, float scale,
                               int32_t ntokens, int32_t topk, int32_t n, void *out, void *stream);
 
@@ -290,6 +296,15 @@ int fluxmi_quant_e4m3_square(const void *x_bf16, int64_t batch, int64_t rows, in
  * ---------------------------------------------------------------------------------------------- */
 int fluxmi_quant_e4m3_block128(const void *x_bf16, int64_t rows, int64_t cols, float eps, void *q_out,
                                float *scale_inv_out, void *q_t_out, float *scale_inv_t_out, void *stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Calibration streams (no counterpart in the reference; for benchmarks): what the memory system of the GPU at
+ * hand gives a kernel that only streams.  copy == 0: every byte of src[0, bytes) is read once (16 bytes per lane
+ * and load, eight loads in flight per lane) and fluxmi_calib_stream_sink_bytes() bytes of dst are written;
+ * copy != 0: the same reads, each stored to dst[0, bytes).  bytes and both pointers are multiples of 16.
+ * ---------------------------------------------------------------------------------------------- */
+size_t fluxmi_calib_stream_sink_bytes(void);
+int fluxmi_calib_stream(const void *src, void *dst, size_t bytes, int32_t copy, void *stream);
 
 #ifdef __cplusplus
 }

@@ -458,3 +458,56 @@ def test_last_round_cut_into_pieces(dtype, row_tiles, what):
     else:
         assert float((out - ref).norm() / ref.norm()) < FP8_FROB
         assert torch.allclose(out, ref, rtol=1e-2, atol=1e-2 * float(ref.abs().max()))
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp8"])
+@pytest.mark.parametrize("ksteps", [1, 2, 19, 35, 36, 37, 56, 57, 75])
+def test_skinny_tail_pieces_same_bits_as_in_place(dtype, ksteps):
+    """Experts whose last row tile holds 1 .. 64 rows: by default (when such tiles are few) that row tile runs behind all
+    other tiles as 64 x 64 pieces on a ring of twenty 8 KiB stages.  Results must be what the oracle says and, bit for
+    bit, what the schedule without skinny tails gives (FLUXMI_SCHED_NO_SKINNY_TAIL = 4; 8 forces them), over K
+    lengths on both sides of the hand-over from the unrolled trips of twenty k-steps to the pair-wise tail (36
+    k-steps), odd numbers of k-steps, with N that is not a multiple of 64, a gather, and every epilogue scale."""
+    from flux_amd import capi
+    elt = 2 if dtype == "bf16" else 1
+    k = ksteps * 64 // elt
+    print(f"[case] grouped_gemm {dtype} skinny tail pieces K={k} ({ksteps} k-steps)", flush=True)
+    g = torch.Generator().manual_seed(100 + ksteps)
+    split = np.array([300, 30, 257, 64, 65, 1, 0, 513, 256], dtype=np.int32)  # skinny: 300, 30, 257, 64, 1, 513
+    rows, n = int(split.sum()), 328
+    src_rows = rows + 37
+    gi = torch.randint(0, src_rows, (rows,), generator=g, dtype=torch.int32)
+    if dtype == "bf16":
+        a = torch.randn(src_rows, k, generator=g).to(torch.bfloat16)
+        w = (torch.randn(len(split), n, k, generator=g) * 0.05).to(torch.bfloat16)
+    else:
+        a = torch.randn(src_rows, k, generator=g).to(torch.float8_e4m3fn)
+        w = (torch.randn(len(split), n, k, generator=g) * 0.25).to(torch.float8_e4m3fn)
+    rs = torch.rand(rows, generator=g) + 0.5
+    cs = torch.rand(len(split), n, generator=g) + 0.5
+    ref = layers.grouped_gemm_fp32(a.float()[gi.long()], w.float(), split, row_scale=rs, col_scale=cs)
+    sp = torch.from_numpy(split).cuda()
+    kw = dict(gather_a=gi.cuda(), row_scale=rs.cuda(), col_scale=cs.cuda())
+    for out_dtype in (torch.bfloat16, torch.float32):
+        base = capi.grouped_gemm(a.cuda(), w.cuda(), sp, out_dtype=out_dtype, sched_flags=4, **kw)
+        for flags in (0, 8):
+            got = capi.grouped_gemm(a.cuda(), w.cuda(), sp, out_dtype=out_dtype, sched_flags=flags, **kw)
+            assert torch.equal(got, base), f"sched_flags={flags} out={out_dtype}: bits differ from the in-place schedule"
+        if out_dtype == torch.float32:
+            assert torch.allclose(base.cpu(), ref, rtol=1e-4, atol=1e-3 * max(1.0, k ** 0.5 * (0.05 if dtype == "bf16" else 1.0)))
+        elif dtype == "bf16":
+            assert_close(base, ref, "skinny")
+        else:
+            assert float((base.float().cpu() - ref).norm() / ref.norm()) < 5e-3
+    # plain (no gather, no scales: the unscaled epilogue), scattered rows, and two weight groups in one launch
+    perm = torch.randperm(rows, generator=g).to(torch.int32).cuda()
+    a2 = a[:rows].cuda()
+    for kw2 in (dict(), dict(scatter_d=perm)):
+        base = capi.grouped_gemm(a2, w.cuda(), sp, sched_flags=4, **kw2)
+        got = capi.grouped_gemm(a2, w.cuda(), sp, sched_flags=8, **kw2)
+        assert torch.equal(got, base)
+    w2 = w.flip(0).contiguous().cuda()
+    outs4 = capi.grouped_gemm_multi(a2, [w.cuda(), w2], sp, sched_flags=4)
+    outs8 = capi.grouped_gemm_multi(a2, [w.cuda(), w2], sp, sched_flags=8)
+    for o4, o8 in zip(outs4, outs8):
+        assert torch.equal(o4, o8)

@@ -268,7 +268,7 @@ def test_profiling_registers_a_schedule_and_keeps_results(c1):
     assert m.num_tuning_records() == 1
     rec = ctx.get_latest_record()
     assert f"experts={e} n={f} k={h} rows={t * k} groups=1" in rec.shape
-    assert rec.raster_rows in (4, 8, 16) and 0 <= rec.sched_flags <= 3
+    assert rec.raster_rows in (4, 8, 16) and rec.sched_flags in (0, 1, 2, 3, 4, 8)
     assert ctx.get_latest_prof_result().count("TopK=") == 5
     assert torch.equal(op0.forward(x, w1, splits_gpu, scatter_index), ref0)  # now under the registered schedule
 
@@ -286,6 +286,15 @@ def test_profiling_registers_a_schedule_and_keeps_results(c1):
     m.load_tuning_record(rec)
     assert m.num_tuning_records() == 1
     m.clear_tuning_records()
+    # the layer1 record also says which form of the top-k reduction won; the text form carries it and loads back
+    rec1 = ctx.get_latest_record()
+    assert rec1.reduce_fused in (False, True)
+    assert ("reduce=fused" in ctx.get_code().splitlines()[-1]) == rec1.reduce_fused
+    assert m.load_tuning_text("fluxmi_gemm_tuning dtype=bf16 experts=%d n=%d k=%d rows=%d groups=1 raster_rows=8 "
+                              "sched_flags=0 reduce=fused\n" % (e, h, f, t * k)) == 1
+    forced = op1.forward_gather_rs(ref0, w2, torch.from_numpy(wl.splits), routing_idx)  # now the fused form
+    assert torch.equal(forced, ref1)  # top-2: same bits either way
+    m.clear_tuning_records()
     # without a context the profiler still runs and registers
     op0.profiling(x, w1, splits_gpu, scatter_index)
     assert m.num_tuning_records() == 1
@@ -293,7 +302,7 @@ def test_profiling_registers_a_schedule_and_keeps_results(c1):
 
 
 @pytest.mark.parametrize("raster_rows,flags,margin", [(4, 0, 0), (16, 1, 0), (8, 2, 0), (1, 3, 0), (8, 0, 40), (8, 0, 255),
-                                                       (8, 0, 1000)])
+                                                       (8, 0, 1000), (8, 4, 0), (8, 8, 0), (2, 9, 5)])
 def test_tile_schedules_and_cu_margin_do_not_change_a_bit(raster_rows, flags, margin):
     """Launch tuning (raster group height, whole tail tiles, no half tiles) and sm_margin move tiles between
     workgroups; every output bit must stay what the default schedule gives."""

@@ -99,7 +99,7 @@ def test_dtype_and_device_checks():
                                  input_dtype=torch.bfloat16)
     assert (args.max_ntokens, args.hidden, args.ffn_hidden, args.nexperts, args.topk) == (16, 64, 128, 4, 2)
     with pytest.raises(RuntimeError, match="unsupported dtype"):
-        bad = flux_amd.MoeArguments(16, 64, 128, 4, 2, torch.float16)
+        bad = flux_amd.MoeArguments(16, 64, 128, 4, 2, torch.float32)
         flux_amd.GemmGroupedV3AGScatter(flux_amd.DistEnvTPWithEP(None, 1), bad)
     with pytest.raises(RuntimeError, match="device tensor"):
         flux_amd.calc_scatter_index(torch.zeros(4, 2, dtype=torch.int32), torch.zeros(4, dtype=torch.int32))
