@@ -237,6 +237,13 @@ def aux_measurements(torch, capi, configs, a, wl, dev, gen, tensors):
     ws = torch.empty(t * h * 4, dtype=torch.uint8, device=dev)
     t_fused = time_loop(torch, lambda: capi.grouped_gemm_topk_reduce(y, w2, sp, tok, t, out=out, workspace=ws,
                                                                      row_scale=row_w), 20)
+    # the same layer with the reference's own data flow: a bf16 intermediate (each top-k term rounded before the sum;
+    # the op's inter_dtype option, tolerance 2e-2 as in the reference's test of that flow)
+    zb16 = torch.empty(m, h, dtype=torch.bfloat16, device=dev)
+    t_two16 = time_loop(torch, lambda: (capi.grouped_gemm(y, w2, sp, out=zb16, row_scale=row_w),
+                                        capi.topk_gather_reduce(zb16, sc, k, out=out)), 20)
+    kernels["layer1_gemm_then_gather_reduce_bf16_intermediate"] = gemm_entry(t_two16, gemm_flops)
+    del zb16
     kernels["layer1_gemm_then_gather_reduce"] = gemm_entry(t_two, gemm_flops)
     kernels["layer1_reduce_fused_in_epilogue"] = gemm_entry(t_fused, gemm_flops)
     del z32, ws
@@ -307,6 +314,9 @@ def aux_measurements(torch, capi, configs, a, wl, dev, gen, tensors):
     f4l = 2.0 * m4 * h4 * f4
     kernels["gemm_bf16_c4_layer0"] = gemm_entry(time_loop(torch, lambda: capi.grouped_gemm(x4, w14, sp4, out=y4, gather_a=gi4), 30), f4l)
     kernels["gemm_bf16_c4_layer1"] = gemm_entry(time_loop(torch, lambda: capi.grouped_gemm(y4, w24, sp4, out=z4, row_scale=rw4), 30), f4l)
+    z4b = torch.empty(m4, h4, dtype=torch.bfloat16, device=dev)
+    kernels["gemm_bf16_c4_layer1_bf16_intermediate"] = gemm_entry(time_loop(torch, lambda: capi.grouped_gemm(y4, w24, sp4, out=z4b, row_scale=rw4), 30), f4l)
+    del z4b
     kernels["gemm_bf16_c4_layer0"]["rows_per_expert_min_max"] = [int(wl4.splits.min()), int(wl4.splits.max())]
     del x4, w14, w24, y4, z4
 
@@ -328,6 +338,11 @@ def aux_measurements(torch, capi, configs, a, wl, dev, gen, tensors):
         sb = torch.rand(e5, n5 // 128, k5 // 128, generator=gen, device=dev) + 0.5
         t_bs = time_loop(torch, lambda: capi.grouped_gemm_blockscale(a8, b8, sp5, sa, sb, out=d5), 20)
         kernels[f"gemm_fp8_blockscale_c5_{tag}"] = gemm_entry(t_bs, f5, PEAK_FP8_TFLOPS, "frac_fp8_peak")
+        # This kernel on the dense problem the library's kernel is timed on below: one weight matrix for all rows
+        # (E = 1, 1/32 of the weight bytes, so the weights stay cache-resident), the like-for-like comparison.
+        sp1 = torch.tensor([m5], dtype=torch.int32, device=dev)
+        t_d1 = time_loop(torch, lambda: capi.grouped_gemm(a8, b8[:1], sp1, out=d5, row_scale=rs5, col_scale=cs5[:1]), 20)
+        kernels[f"gemm_fp8_dense_one_weight_c5_{tag}"] = gemm_entry(t_d1, f5, PEAK_FP8_TFLOPS, "frac_fp8_peak")
         # The library's fp8 GEMM (torch._scaled_mm = hipBLASLt) for scale: the same work as a loop of per-expert
         # GEMMs, and one dense GEMM of the same FLOPs with a single weight matrix (1/32 of the weight bytes).
         try:

@@ -56,15 +56,17 @@ __device__ __forceinline__ Vec8<IN_F32> zero8() {
   return r;
 }
 
-// f16 (wave-uniform): 16-bit inputs are fp16 instead of bf16; fp32 inputs ignore it.
-__device__ __forceinline__ void accumulate8(float (&acc)[8], const Vec8<true> &x, const float w, bool) {
+// F16: 16-bit inputs are fp16 instead of bf16; fp32 inputs ignore it.
+template <bool F16>
+__device__ __forceinline__ void accumulate8(float (&acc)[8], const Vec8<true> &x, const float w) {
 #pragma unroll
   for (int i = 0; i < 8; ++i) acc[i] = fmaf(w, __uint_as_float(x.v[i >> 2][i & 3]), acc[i]);
 }
 
-__device__ __forceinline__ void accumulate8(float (&acc)[8], const Vec8<false> &x, const float w, bool f16) {
+template <bool F16>
+__device__ __forceinline__ void accumulate8(float (&acc)[8], const Vec8<false> &x, const float w) {
   const u32x4 v = x.v[0];
-  if (f16) {
+  if constexpr (F16) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const uint32_t u = v[i];
@@ -87,19 +89,20 @@ __device__ __forceinline__ bool row_in_range(int32_t r, int32_t nrows) {
   return static_cast<uint32_t>(r) < static_cast<uint32_t>(nrows);
 }
 
-// Two results to the packed 16-bit output type: bf16, or fp16 when f16 (wave-uniform) is set.
-__device__ __forceinline__ uint32_t pack2(float lo, float hi, bool f16) {
-  if (f16) return static_cast<uint32_t>(float_to_f16_bits(lo)) | (static_cast<uint32_t>(float_to_f16_bits(hi)) << 16);
+// Two results to the packed 16-bit output type: bf16, or fp16.
+template <bool F16>
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+  if constexpr (F16) return static_cast<uint32_t>(float_to_f16_bits(lo)) | (static_cast<uint32_t>(float_to_f16_bits(hi)) << 16);
   return static_cast<uint32_t>(float_to_bf16_bits(lo)) | (static_cast<uint32_t>(float_to_bf16_bits(hi)) << 16);
 }
 
 // TOPK > 0: compile-time top-k (loads fully unrolled).  TOPK == 0: run-time top-k.
 // NT: non-temporal source loads.  The choice is made once per launch and hoisted out of the load
 // sequence, so that no control flow sits between the loads of one output vector.
-template <int TOPK, int NGROUPS, bool WEIGHTED, bool IN_F32, bool NT>
+template <int TOPK, int NGROUPS, bool WEIGHTED, bool IN_F32, bool NT, bool F16>
 __device__ __forceinline__ void topk_gather_reduce_body(
     const GroupPtrs &in, const int32_t *__restrict__ routing_idx, const float *__restrict__ row_weight,
-    float scale, int32_t topk_rt, int32_t nvec, int32_t nrows, bool f16, uint16_t *__restrict__ out) {
+    float scale, int32_t topk_rt, int32_t nvec, int32_t nrows, uint16_t *__restrict__ out) {
   const int t = blockIdx.x;
   const int topk = TOPK > 0 ? TOPK : topk_rt;
   const size_t row_vecs = static_cast<size_t>(nvec);
@@ -144,14 +147,14 @@ __device__ __forceinline__ void topk_gather_reduce_body(
       u32x2 *dst = reinterpret_cast<u32x2 *>(out) + static_cast<size_t>(t) * nq;
       if (oka) {
         u32x2 o;
-        o[0] = pack2(a[0] * scale, a[1] * scale, f16);
-        o[1] = pack2(a[2] * scale, a[3] * scale, f16);
+        o[0] = pack2<F16>(a[0] * scale, a[1] * scale);
+        o[1] = pack2<F16>(a[2] * scale, a[3] * scale);
         __builtin_nontemporal_store(o, dst + qa);
       }
       if (okb) {
         u32x2 o;
-        o[0] = pack2(b[0] * scale, b[1] * scale, f16);
-        o[1] = pack2(b[2] * scale, b[3] * scale, f16);
+        o[0] = pack2<F16>(b[0] * scale, b[1] * scale);
+        o[1] = pack2<F16>(b[2] * scale, b[3] * scale);
         __builtin_nontemporal_store(o, dst + qb);
       }
     }
@@ -178,7 +181,7 @@ __device__ __forceinline__ void topk_gather_reduce_body(
 #pragma unroll
       for (int g = 0; g < NGROUPS; ++g) {
 #pragma unroll
-        for (int j = 0; j < TOPK; ++j) accumulate8(acc, vals[g][j], w[j], f16);
+        for (int j = 0; j < TOPK; ++j) accumulate8<F16>(acc, vals[g][j], w[j]);
       }
     } else {
       for (int g = 0; g < NGROUPS; ++g) {
@@ -186,37 +189,37 @@ __device__ __forceinline__ void topk_gather_reduce_body(
           const int32_t r = routing_idx[static_cast<size_t>(t) * topk + j];
           if (!row_in_range(r, nrows)) continue;
           const float w = WEIGHTED ? row_weight[r] : 1.f;
-          accumulate8(acc, load8<IN_F32, NT>(in.p[g], static_cast<size_t>(r), row_vecs, v), w, f16);
+          accumulate8<F16>(acc, load8<IN_F32, NT>(in.p[g], static_cast<size_t>(r), row_vecs, v), w);
         }
       }
     }
     u32x4 o;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) o[i] = pack2(acc[2 * i] * scale, acc[2 * i + 1] * scale, f16);
+    for (int i = 0; i < 4; ++i) o[i] = pack2<F16>(acc[2 * i] * scale, acc[2 * i + 1] * scale);
     u32x4 *dst = reinterpret_cast<u32x4 *>(out) + static_cast<size_t>(t) * row_vecs + v;
     __builtin_nontemporal_store(o, dst);
   }
 }
 
-template <int TOPK, int NGROUPS, bool WEIGHTED, bool IN_F32>
+template <int TOPK, int NGROUPS, bool WEIGHTED, bool IN_F32, bool F16>
 __global__ __launch_bounds__(kMaxThreads) void topk_gather_reduce_kernel(
     GroupPtrs in, const int32_t *__restrict__ routing_idx, const float *__restrict__ row_weight,
-    float scale, int32_t topk_rt, int32_t nvec /* n / 8 */, int32_t nrows, int32_t flags /* 1: non-temporal loads, 2: fp16 */,
+    float scale, int32_t topk_rt, int32_t nvec /* n / 8 */, int32_t nrows, int32_t nt_loads,
     uint16_t *__restrict__ out) {
-  const bool f16 = (flags & 2) != 0;
-  if (flags & 1)
-    topk_gather_reduce_body<TOPK, NGROUPS, WEIGHTED, IN_F32, true>(in, routing_idx, row_weight, scale, topk_rt,
-                                                                   nvec, nrows, f16, out);
+  if (nt_loads)
+    topk_gather_reduce_body<TOPK, NGROUPS, WEIGHTED, IN_F32, true, F16>(in, routing_idx, row_weight, scale, topk_rt,
+                                                                        nvec, nrows, out);
   else
-    topk_gather_reduce_body<TOPK, NGROUPS, WEIGHTED, IN_F32, false>(in, routing_idx, row_weight, scale, topk_rt,
-                                                                    nvec, nrows, f16, out);
+    topk_gather_reduce_body<TOPK, NGROUPS, WEIGHTED, IN_F32, false, F16>(in, routing_idx, row_weight, scale, topk_rt,
+                                                                         nvec, nrows, out);
 }
 
-template <int TOPK, int NGROUPS>
+// F16 (fp16 inputs and / or output) exists for the run-time top-k form only: the unrolled forms are the bf16 path's.
+template <int TOPK, int NGROUPS, bool F16 = false>
 void launch(bool weighted, bool in_f32, dim3 grid, int threads, int nt, hipStream_t s, const GroupPtrs &in,
             const int32_t *idx, const float *w, float scale, int32_t topk, int32_t nvec, int32_t nrows, uint16_t *out) {
-#define FLUXMI_GR_LAUNCH(W, F)                                                                       \
-  hipLaunchKernelGGL((topk_gather_reduce_kernel<TOPK, NGROUPS, W, F>), grid, dim3(threads), 0, s, in, \
+#define FLUXMI_GR_LAUNCH(W, F)                                                                            \
+  hipLaunchKernelGGL((topk_gather_reduce_kernel<TOPK, NGROUPS, W, F, F16>), grid, dim3(threads), 0, s, in, \
                      idx, w, scale, topk, nvec, nrows, nt, out)
   if (weighted) {
     if (in_f32) FLUXMI_GR_LAUNCH(true, true);
@@ -230,7 +233,11 @@ void launch(bool weighted, bool in_f32, dim3 grid, int threads, int nt, hipStrea
 
 template <int NGROUPS>
 void dispatch_topk(bool weighted, bool in_f32, dim3 grid, int threads, int nt, hipStream_t s, const GroupPtrs &in, const int32_t *idx,
-                   const float *w, float scale, int32_t topk, int32_t nvec, int32_t nrows, uint16_t *out) {
+                   const float *w, float scale, int32_t topk, int32_t nvec, int32_t nrows, uint16_t *out, bool f16) {
+  if (f16) {
+    launch<0, NGROUPS, true>(weighted, in_f32, grid, threads, nt, s, in, idx, w, scale, topk, nvec, nrows, out);
+    return;
+  }
   switch (topk) {
     case 1: launch<1, NGROUPS>(weighted, in_f32, grid, threads, nt, s, in, idx, w, scale, topk, nvec, nrows, out); break;
     case 2: launch<2, NGROUPS>(weighted, in_f32, grid, threads, nt, s, in, idx, w, scale, topk, nvec, nrows, out); break;
@@ -254,7 +261,7 @@ extern "C" int fluxmi_topk_gather_reduce(const void *const *in, int32_t ngroups,
   FLUXMI_REQUIRE(io_format >= 0 && io_format <= 3, FLUXMI_ERR_INVALID_ARG,
                  "topk_gather_reduce: io_format=%d outside [0,3]", io_format);
   const int32_t in_fp32 = io_format & 1;
-  const int32_t half_f16 = (io_format & 2) ? 2 : 0;
+  const bool half_f16 = (io_format & 2) != 0;
   FLUXMI_REQUIRE(ngroups >= 1 && ngroups <= kMaxGroups, FLUXMI_ERR_UNSUPPORTED,
                  "topk_gather_reduce: ngroups=%d outside [1,%d]", ngroups, kMaxGroups);
   FLUXMI_REQUIRE(topk >= 1 && topk <= 64, FLUXMI_ERR_UNSUPPORTED,
@@ -286,16 +293,16 @@ extern "C" int fluxmi_topk_gather_reduce(const void *const *in, int32_t ngroups,
     if (ysplit > 16) ysplit = 16;
   }
   const size_t in_bytes = static_cast<size_t>(ntokens) * topk * n * (in_fp32 ? 4 : 2) * ngroups;
-  const int nt = (in_bytes > kPlainLoadMaxBytes ? 1 : 0) | half_f16;
+  const int nt = in_bytes > kPlainLoadMaxBytes ? 1 : 0;
   const dim3 grid(static_cast<unsigned>(ntokens), static_cast<unsigned>(ysplit));
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool weighted = row_weight != nullptr;
   uint16_t *o = static_cast<uint16_t *>(out);
   switch (ngroups) {
-    case 1: dispatch_topk<1>(weighted, in_fp32 != 0, grid, threads, nt, s, gp, routing_idx, row_weight, scale, topk, nvec, nrows, o); break;
-    case 2: dispatch_topk<2>(weighted, in_fp32 != 0, grid, threads, nt, s, gp, routing_idx, row_weight, scale, topk, nvec, nrows, o); break;
-    case 3: dispatch_topk<3>(weighted, in_fp32 != 0, grid, threads, nt, s, gp, routing_idx, row_weight, scale, topk, nvec, nrows, o); break;
-    default: dispatch_topk<4>(weighted, in_fp32 != 0, grid, threads, nt, s, gp, routing_idx, row_weight, scale, topk, nvec, nrows, o); break;
+    case 1: dispatch_topk<1>(weighted, in_fp32 != 0, grid, threads, nt, s, gp, routing_idx, row_weight, scale, topk, nvec, nrows, o, half_f16); break;
+    case 2: dispatch_topk<2>(weighted, in_fp32 != 0, grid, threads, nt, s, gp, routing_idx, row_weight, scale, topk, nvec, nrows, o, half_f16); break;
+    case 3: dispatch_topk<3>(weighted, in_fp32 != 0, grid, threads, nt, s, gp, routing_idx, row_weight, scale, topk, nvec, nrows, o, half_f16); break;
+    default: dispatch_topk<4>(weighted, in_fp32 != 0, grid, threads, nt, s, gp, routing_idx, row_weight, scale, topk, nvec, nrows, o, half_f16); break;
   }
   FLUXMI_HIP_CHECK(hipGetLastError());
   return FLUXMI_OK;

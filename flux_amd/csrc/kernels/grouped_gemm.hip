@@ -68,7 +68,9 @@ __global__ __launch_bounds__(256) void grouped_gemm_generic_kernel(const GemmPar
                                          static_cast<int64_t>(kb) * (s_row_off[e + 1] - s_row_off[e]) + (r - s_row_off[e])];
         const float bs = p.b_scale_layout == FLUXMI_BSCALE_N_K
                              ? p.b_scale[(static_cast<int64_t>(e) * nblocks + nb) * kblocks + kb]
-                             : p.b_scale[(static_cast<int64_t>(e) * kblocks + kb) * nblocks + nb];
+                             : p.b_scale_layout == FLUXMI_BSCALE_K_N
+                                   ? p.b_scale[(static_cast<int64_t>(e) * kblocks + kb) * nblocks + nb]
+                                   : p.b_scale[((static_cast<int64_t>(e) * nblocks + nb) * kblocks + kb) * 128 + (n & 127)];
         total = fmaf(acc, as * bs, total);
         acc = 0.f;
       }
@@ -178,11 +180,13 @@ int run_grouped_gemm(const fluxmi_grouped_gemm_args *args, int ngroups, const vo
     FLUXMI_REQUIRE(bs->a_scale != nullptr && bs->b_scale != nullptr, FLUXMI_ERR_INVALID_ARG,
                    "grouped_gemm_blockscale: null a_scale / b_scale");
     FLUXMI_REQUIRE((bs->a_layout == FLUXMI_ASCALE_BLOCK128 || bs->a_layout == FLUXMI_ASCALE_EXPERT_K_M) &&
-                       (bs->b_layout == FLUXMI_BSCALE_N_K || bs->b_layout == FLUXMI_BSCALE_K_N),
+                       (bs->b_layout == FLUXMI_BSCALE_N_K || bs->b_layout == FLUXMI_BSCALE_K_N ||
+                        bs->b_layout == FLUXMI_BSCALE_COL_N_K),
                    FLUXMI_ERR_INVALID_ARG, "grouped_gemm_blockscale: unknown scale layout (%d, %d)", bs->a_layout, bs->b_layout);
     FLUXMI_REQUIRE(!(bs->a_layout == FLUXMI_ASCALE_EXPERT_K_M && args->gather_a != nullptr), FLUXMI_ERR_INVALID_ARG,
                    "grouped_gemm_blockscale: per-expert a_scale segments cannot be combined with gather_a");
     FLUXMI_REQUIRE(ngroups == 1, FLUXMI_ERR_UNSUPPORTED, "grouped_gemm_blockscale: one weight tensor per launch");
+    if (bs->b_layout == FLUXMI_BSCALE_COL_N_K) mfma = false;  // per-column weight scales: the generic kernel only
     // a_scale is addressed with 32-bit byte offsets
     const int64_t srows = args->gather_a ? args->a_rows : args->max_rows;
     mfma = mfma && ((srows + 127) / 128 * 128) * (args->k / 128) * 4 < (int64_t{1} << 32) &&

@@ -137,7 +137,12 @@ static torch::Tensor blockscale_run(const torch::Tensor &input, const torch::Ten
   // The layout is taken from the rank, so the shape has to be exactly that layout's: a tensor of the right size in
   // another arrangement (a [E, K/128, N/128] weight scale, a natural [M, K/128] input scale) would be read wrongly
   // without any error.
-  if (b_layout == FLUXMI_BSCALE_N_K) {
+  if (b_layout == FLUXMI_BSCALE_COL_N_K) {
+    TORCH_CHECK(weight_scale.dim() == 4 && weight_scale.size(0) == e && weight_scale.size(1) == nb && weight_scale.size(2) == kb &&
+                    weight_scale.size(3) == kBlock,
+                "per-column weight_scale must be [ceil(N/128), K/128, 128] = [", nb, ", ", kb, ", ", kBlock, "]; got ",
+                weight_scale.sizes());
+  } else if (b_layout == FLUXMI_BSCALE_N_K) {
     TORCH_CHECK(weight_scale.dim() == 3 && weight_scale.size(0) == e && weight_scale.size(1) == nb && weight_scale.size(2) == kb,
                 "weight_scale must be a 3-D tensor [E, ceil(N/128), K/128] = [", e, ", ", nb, ", ", kb,
                 "] (as Quantization returns it) or the reference's flat 1-D [E * K/128 * N/128]; got ", weight_scale.sizes());
@@ -256,14 +261,26 @@ torch::Tensor BlockScaleGemm::forward_multistream(torch::Tensor input, torch::Te
                         FLUXMI_BSCALE_N_K, output_dtype_);
 }
 
-// The reference's second implementation of forward (blockscale_gemm.cc:954-973); one kernel serves both here.  Its
-// per-column form of the weight scales is not built.
+// The reference's second implementation of forward (blockscale_gemm.cc:954-973); one kernel serves both here.  With
+// is_groupwise_b the weight carries one scale per column and 128 of K, [ceil(N/128), K/128, 128] (the
+// ScaleNsPerTile == BLOCK_N case of test/python/gemm_only/test_blockwise_scale_gemm_only.py:209,237-240): that form
+// runs on the generic kernel (a checking path, as `reference` is in the reference).
 torch::Tensor BlockScaleGemm::reference(torch::Tensor input, torch::Tensor weight, std::optional<torch::Tensor> bias,
                                         std::optional<torch::Tensor> output, std::optional<torch::Tensor> input_scale,
                                         std::optional<torch::Tensor> weight_scale, bool is_groupwise_b) {
-  TORCH_CHECK(!is_groupwise_b, "BlockScaleGemm.reference: per-column weight scales (is_groupwise_b) are not supported");
-  return forward(std::move(input), std::move(weight), std::move(bias), std::move(output), std::move(input_scale),
-                 std::move(weight_scale));
+  if (!is_groupwise_b)
+    return forward(std::move(input), std::move(weight), std::move(bias), std::move(output), std::move(input_scale),
+                   std::move(weight_scale));
+  TORCH_CHECK(!bias.has_value(), "BlockScaleGemm: bias is not supported");
+  TORCH_CHECK(input_scale.has_value() && weight_scale.has_value(), "BlockScaleGemm: input_scale and weight_scale are required");
+  FLUX_AMD_CHECK_INPUT(input, input_dtype_);
+  FLUX_AMD_CHECK_INPUT(weight, weight_dtype_);
+  FLUX_AMD_CHECK_NDIM(input, 2);
+  FLUX_AMD_CHECK_NDIM(weight, 2);
+  TORCH_CHECK(weight_scale->dim() == 3, "per-column weight_scale must be [ceil(N/128), K/128, 128], got ", weight_scale->sizes());
+  torch::Tensor splits = torch::full({1}, input.size(0), at::TensorOptions().dtype(at::kInt));
+  return blockscale_run(input, weight.unsqueeze(0), splits, output, *input_scale, FLUXMI_ASCALE_BLOCK128,
+                        weight_scale->unsqueeze(0), FLUXMI_BSCALE_COL_N_K, output_dtype_);
 }
 
 // The reference times every registered kernel configuration and runs the best (blockscale_gemm.cc:975-1023); there is

@@ -82,10 +82,29 @@ PYBIND11_MODULE(flux_ths_pybind, m) {
            py::arg("fast_accum") = false, py::arg("sm_margin") = 0, py::arg("prof_ctx") = nullptr);
 
   py::class_<GemmGroupedV3GatherRS>(m, "GemmGroupedV3GatherRS")
-      .def(py::init<int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, bool>(),
+      // The reference's ten arguments (src/pybind/gemm_grouped_v3_gather_rs.cc:36-50) and, after them, one of this
+      // build: the dtype of the [M, N] intermediate between the GEMM and the top-k reduction.  None / torch.float32
+      // (default): one rounding in the whole layer; the 16-bit output type (torch.bfloat16 / torch.float16): the
+      // reference's own data flow (its inter_D), each top-k term rounded before the sum, half the intermediate's
+      // bytes, the reference's own 2e-2 test bound.  $FLUX_AMD_INTER_DTYPE=bf16 sets the default to the latter.
+      .def(py::init([](int64_t total_num_experts, int64_t max_m, int64_t n_dim, int64_t topk, int64_t rank,
+                       int64_t world_size, int64_t tp_world_size, int64_t ep_world_size, int64_t max_input_groups,
+                       bool ep_in_dp, py::object inter_dtype) {
+             auto *op = new GemmGroupedV3GatherRS(total_num_experts, max_m, n_dim, topk, rank, world_size, tp_world_size,
+                                                  ep_world_size, max_input_groups, ep_in_dp);
+             if (!inter_dtype.is_none()) {
+               const at::ScalarType t = to_dtype(inter_dtype);
+               if (t != at::kFloat && t != at::kBFloat16 && t != at::kHalf) {
+                 delete op;
+                 TORCH_CHECK(false, "inter_dtype must be torch.float32 or the 16-bit output type, got ", t);
+               }
+               op->set_intermediate_fp32(t == at::kFloat);
+             }
+             return op;
+           }),
            py::arg("total_num_experts"), py::arg("max_m"), py::arg("n_dim"), py::arg("topk"), py::arg("rank"),
            py::arg("world_size"), py::arg("tp_world_size"), py::arg("ep_world_size"),
-           py::arg("max_input_groups") = 1, py::arg("ep_in_dp") = false)
+           py::arg("max_input_groups") = 1, py::arg("ep_in_dp") = false, py::arg("inter_dtype") = py::none())
       .def("forward_gather_rs", &GemmGroupedV3GatherRS::forward_gather_rs, py::arg("input"), py::arg("weight"),
            py::arg("splits_cpu"), py::arg("routing_idx"), py::arg("n_tokens_per_rank") = py::none(),
            py::arg("input_scale") = py::none(), py::arg("weight_scale") = py::none(),

@@ -73,6 +73,16 @@ class GemmGroupedV3GatherRS {
   void lazy_init(const torch::Tensor &like);
   int64_t num_experts_, max_m_, n_dim_, topk_, max_input_groups_;
   bool inter_fp32_ = true;
+
+ public:
+  // Dtype of the intermediate between the GEMM and the reduction: fp32 (one rounding in the layer) or the 16-bit
+  // output type (the reference's inter_D).  Only before the first forward: the buffers are allocated lazily.
+  void set_intermediate_fp32(bool fp32) {
+    TORCH_CHECK(inter_.empty(), "the intermediate's dtype is fixed once the op has run");
+    inter_fp32_ = fp32;
+  }
+
+ private:
   int fused_mode_ = 0;  // 0: by shape, 1: always the fused epilogue reduce, 2: always GEMM + gather-reduce
   std::vector<torch::Tensor> inter_;
   torch::Tensor splits_dev_;

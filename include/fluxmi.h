@@ -146,7 +146,7 @@ typedef struct fluxmi_grouped_gemm_args {
 #define FLUXMI_SCHED_WHOLE_TAIL_TILES 1 /* do not cut the tiles of the last, partly filled round into pieces */
 #define FLUXMI_SCHED_NO_HALF_TILES 2    /* run the last row tile of an expert 256 rows high even if 128 cover it, and the last column tile 256 wide even if 128 cover it */
 #define FLUXMI_SCHED_NO_SKINNY_TAIL 4    /* never move the last row tiles of experts that hold at most 64 rows behind all other tiles as 64 x 64 pieces */
-#define FLUXMI_SCHED_FORCE_SKINNY_TAIL 8 /* always do so (by default only when those pieces fill at most two rounds of the launch) */
+#define FLUXMI_SCHED_FORCE_SKINNY_TAIL 8 /* always do so (by default only when those pieces fill at most two rounds of the launch and K spans at least 128 steps of 64 bytes) */
 
 size_t fluxmi_grouped_gemm_workspace_bytes(const fluxmi_grouped_gemm_args *args);
 int fluxmi_grouped_gemm(const fluxmi_grouped_gemm_args *args, void *workspace,
@@ -206,6 +206,9 @@ int fluxmi_grouped_gemm_topk_reduce(const fluxmi_grouped_gemm_args *args, const 
 #define FLUXMI_ASCALE_EXPERT_K_M 1
 #define FLUXMI_BSCALE_N_K 0
 #define FLUXMI_BSCALE_K_N 1
+#define FLUXMI_BSCALE_COL_N_K 2 /* one scale per column of B and 128 of K: [E, ceil(N / 128), K / 128, 128], column
+                                   inside its block fastest (the `is_groupwise_b` form of BlockScaleGemm::reference,
+                                   src/comm_none/ths_op/blockscale_gemm.cc:954-973); served by the generic kernel */
 int fluxmi_grouped_gemm_blockscale(const fluxmi_grouped_gemm_args *args, const float *a_scale,
                                    int32_t a_scale_layout, const float *b_scale, int32_t b_scale_layout,
                                    void *stream);

@@ -368,7 +368,16 @@ def test_blockscale_gemm_op_dense_and_grouped():
     # the reference's second implementation and its tuning entry point: one kernel here
     assert torch.equal(op.reference(qx, qw[0], input_scale=sx, weight_scale=sw[0].contiguous()), d)
     assert torch.equal(op.profiling(qx, qw[0], input_scale=sx, weight_scale=sw[0].contiguous()), d)
-    with pytest.raises(RuntimeError, match="is_groupwise_b"):
+    # is_groupwise_b: one weight scale per column and 128 of K, [N/128, K/128, 128] (test_blockwise_scale_gemm_only.py:209,
+    # 237-240); the oracle is the same dequantise-matmul with the scale taken per column
+    gq = torch.Generator().manual_seed(13)
+    swc = (torch.rand(n // 128, k // 128, 128, generator=gq) + 0.5) * float(sw[0].mean())
+    dq = op.reference(qx, qw[0], input_scale=sx, weight_scale=swc.cuda(), is_groupwise_b=True)
+    wq = qw[0].cpu().float().reshape(n // 128, 128, k // 128, 128) * swc.permute(0, 2, 1)[:, :, :, None]
+    aq = qx.cpu().float().reshape(m, k // 128, 128) * sa[:, :, None]
+    refq = aq.reshape(m, k) @ wq.reshape(n, k).t()
+    assert torch.allclose(dq.float().cpu(), refq, rtol=1e-2, atol=1e-2 * float(refq.abs().max()))
+    with pytest.raises(RuntimeError, match="per-column weight_scale"):
         op.reference(qx, qw[0], input_scale=sx, weight_scale=sw[0].contiguous(), is_groupwise_b=True)
     with pytest.raises(RuntimeError, match="bias"):
         op.forward(qx, qw[0], bias=torch.zeros(1, device="cuda"), input_scale=sx, weight_scale=sw[0].contiguous())
@@ -411,3 +420,27 @@ def test_layer1_op_with_the_fused_epilogue_reduce(c1, monkeypatch):
     monkeypatch.setenv("FLUX_AMD_LAYER1_REDUCE", "sideways")
     with pytest.raises(RuntimeError, match="FLUX_AMD_LAYER1_REDUCE"):
         flux_amd.GemmGroupedV3GatherRS(e, t * k, h, k, 0, 1, 1, 1)
+
+
+def test_layer1_intermediate_dtype_is_a_constructor_option(c1):
+    """inter_dtype (after the reference's ten constructor arguments): fp32 by default, the 16-bit output type on
+    request — the reference's own data flow, checked at the reference's own bound for it (2e-2 / 2e-2,
+    test/python/moe_gather_rs/test_moe_gather_rs.py:397-411)."""
+    wl = c1
+    t, k, e, h, f = wl.tokens, wl.topk, wl.experts, wl.hidden, wl.ffn
+    y = layers.layer0_fp32(wl.tensors["x"], wl.tensors["w1"], wl.splits, wl.gather_index).to(torch.bfloat16).cuda()
+    w2 = wl.tensors["w2"].cuda()
+    idx = torch.from_numpy(wl.scatter_index.reshape(-1)).cuda()
+    ovs = wl.row_weight.cuda()
+    ref = layers.layer1_fp32(y.cpu(), wl.tensors["w2"], wl.splits, wl.scatter_index.reshape(-1), k, output_vec_scale=wl.row_weight)
+    outs = {}
+    for name, dt in (("default", None), ("fp32", torch.float32), ("bf16", torch.bfloat16)):
+        op = flux_amd.GemmGroupedV3GatherRS(e, t * k, h, k, 0, 1, 1, 1, inter_dtype=dt)
+        outs[name] = op.forward_gather_rs(y, w2, torch.from_numpy(wl.splits), idx, output_vec_scale=ovs)
+    assert torch.equal(outs["default"], outs["fp32"])
+    close(outs["fp32"], ref)
+    got = outs["bf16"].float().cpu()
+    assert torch.allclose(got, ref, rtol=2e-2, atol=2e-2), float((got - ref).abs().max())
+    assert not torch.equal(outs["bf16"], outs["fp32"])  # the terms really were rounded before the sum
+    with pytest.raises(RuntimeError, match="inter_dtype"):
+        flux_amd.GemmGroupedV3GatherRS(e, t * k, h, k, 0, 1, 1, 1, inter_dtype=torch.int32)
