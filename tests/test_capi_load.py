@@ -50,6 +50,14 @@ def test_argument_errors_without_gpu():
     assert rc == -1 and b"dtype" in lib.fluxmi_last_error()
     args = capi.GroupedGemmArgs(dtype=0, nexperts=5000, max_rows=1, n=8, k=64)
     assert lib.fluxmi_grouped_gemm(ctypes.byref(args), None, 0, None) == -2
+    args = capi.GroupedGemmArgs(dtype=2, nexperts=2, max_rows=1, n=8, k=64, sched_flags=16)   # fp16 is a dtype; flag 16 is not
+    rc = lib.fluxmi_grouped_gemm(ctypes.byref(args), None, 0, None)
+    assert rc == -1 and b"null a / b / d / splits" in lib.fluxmi_last_error()
+    rc = lib.fluxmi_topk_gather_reduce(ptrs, 1, 4, ctypes.c_void_p(0x1000), None, 1.0, 4, 2, 64, ctypes.c_void_p(0x1000), None)
+    assert rc == -1 and b"io_format" in lib.fluxmi_last_error()
+    rc = lib.fluxmi_calib_stream(ctypes.c_void_p(0x1000), ctypes.c_void_p(0x1000), 24, 0, None)
+    assert rc == -1 and b"multiples of 16" in lib.fluxmi_last_error()
+    assert lib.fluxmi_version() >= 110
 
 
 def test_golden_routing_fixture_matches_oracle():

@@ -130,6 +130,13 @@ def test_tuning_text_round_trip_and_errors():
                       ("fluxmi_gemm_tuning dtype=bf16 experts=1 n=1 k=1 rows=1 groups=1 raster_rows=1 sched_flags=64", "out of range")):
         with pytest.raises(RuntimeError, match=what):
             m.load_tuning_text("# first line\n" + bad)
+    # fp16 shapes, the newer schedule flags and the form of layer1's reduction are part of the text form
+    assert m.load_tuning_text("fluxmi_gemm_tuning dtype=f16 experts=8 n=4096 k=14336 rows=16384 groups=1 raster_rows=8 "
+                              "sched_flags=8 reduce=fused\n"
+                              "fluxmi_gemm_tuning dtype=bf16 experts=8 n=4096 k=14336 rows=16384 groups=1 raster_rows=8 "
+                              "sched_flags=4 reduce=twopass\n") == 2
+    with pytest.raises(RuntimeError, match="unknown reduce form"):
+        m.load_tuning_text("fluxmi_gemm_tuning dtype=bf16 experts=1 n=1 k=1 rows=1 groups=1 raster_rows=1 sched_flags=0 reduce=maybe")
     m.clear_tuning_records()
     assert m.num_tuning_records() == 0
     ctx = m.ProfilingContext("empty")
