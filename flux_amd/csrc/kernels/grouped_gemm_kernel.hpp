@@ -377,8 +377,8 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const uint8_t *base,
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(base), 0, static_cast<int>(n), 0x00020000);
 }
 // Where a work item lies.  kind: 0 a whole macro tile (4, 4); 1 the 128-row tile ending an expert (2, 4);
-// 2 a 256x128 piece (4, 2); 3 a 128x128 piece (2, 2); 4 a 64x64 piece of an expert's last rows (1, 1); -1 an item
-// without work; -2 past the last item.
+// 2 a 256x128 piece (4, 2); 3 a 128x128 piece (2, 2); 4 a 64x64 piece of an expert's last rows (1, 1); 5 the 64-row
+// tile ending an expert (1, 4); -1 an item without work; -2 past the last item.
 // n0 is a column of the launch's virtual output: weight group g (a launch may multiply the same rows by up
 // to four weight tensors, each with an output of its own) occupies columns [g * npad, g * npad + n), npad =
 // n rounded up to whole macro tiles.
@@ -407,8 +407,8 @@ __device__ __forceinline__ int split_group(int &n0, int n, int ngroups) {
 // 8 KiB per stage: twenty stages, sixteen steps ahead, unrolled over twenty k-steps.
 template <int MB, int NB>
 struct Ring {
-  static_assert(MB != 1 || NB == 1, "64-row tiles exist as 64x64 pieces only");
-  static constexpr bool tiny = MB == 1;
+  static_assert(MB != 1 || NB == 1 || NB == 4, "64-row tiles exist as 64x64 pieces and as 64x256 tiles");
+  static constexpr bool tiny = MB == 1 && NB == 1;
   static constexpr bool deep = MB == 2 && NB == 2;
   static constexpr int STG = tiny ? 4 * STAGES : (deep ? 2 * STAGES : STAGES);
   static constexpr int XB = tiny ? X_TILE_BYTES / 4 : (deep ? X_TILE_BYTES / 2 : X_TILE_BYTES);  // X part of a stage
@@ -572,6 +572,9 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
   constexpr int HALF = LOADS;      // ... of which the pair's first step issues this many
   constexpr int WAIT_EVEN = (LA - 2) / 2 * PAIR;  // outstanding fills allowed when an even step starts
   constexpr int WAIT_ODD = (LA - 4) / 2 * PAIR + HALF;
+  // A fill's M0 write is set apart from its load (one MFMA slot ahead) only while every fill of a pair of steps has
+  // an MFMA slot of its own; with more fills than slots (fp8 tiles 64 rows high) the whole fill stays in one place.
+  constexpr bool SPLIT_M0 = LOADS <= NM;
   const int wave = c.wave, lane = c.lane, wm = c.wm, wn = c.wn, nk = c.nk;
   const int e = t.e, row_base = t.row_base, rows_e = t.rows_e, m0 = t.m0;
 
@@ -728,7 +731,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
         constexpr int d = decltype(D)::value;
         constexpr int at = (d * (2 * NM) / (2 * LOADS) + 1) % (2 * NM);
         if constexpr (at == t + (even ? 0 : NM)) {
-          if constexpr (at % NM != 0)  // the slot before is in the same step: M0 was written there
+          if constexpr (SPLIT_M0 && at % NM != 0)  // the slot before is in the same step: M0 was written there
             fill_go(std::integral_constant<int, (d >> 1)>{}, kbase + (e0 + LA + (d & 1)) * KBYTES);
           else
             fill_one(std::integral_constant<int, (e0 + LA + (d & 1)) % STG>{}, std::integral_constant<int, (d >> 1)>{},
@@ -738,7 +741,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
       static_for<0, 2 * LOADS>([&](auto D) {
         constexpr int d = decltype(D)::value;
         constexpr int at = (d * (2 * NM) / (2 * LOADS) + 1) % (2 * NM);
-        if constexpr (at % NM != 0 && at - 1 == t + (even ? 0 : NM))
+        if constexpr (SPLIT_M0 && at % NM != 0 && at - 1 == t + (even ? 0 : NM))
           fill_m0(std::integral_constant<int, (e0 + LA + (d & 1)) % STG>{}, std::integral_constant<int, (d >> 1)>{});
       });
       mfma_slot<ELT, MBK, NBK>(t, xc, wc, acc);
@@ -1303,9 +1306,10 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
     if (item < full_items || pieces == 1) {
       // The last row tile of an expert is run 128 rows high when that covers its rows, the last column
       // tile 128 columns wide when that covers its columns (N = 1408: the sixth tile holds 128 columns).
+      // With at most 64 rows left (and the skinny tail not in use for them) it runs 64 rows high.
       const bool low = half_tiles && rows_e - t.m0 <= 128;
       const bool narrow = half_tiles && p.n - t.n0 <= 128;
-      t.kind = low ? (narrow ? 3 : 1) : (narrow ? 2 : 0);
+      t.kind = low ? (narrow ? 3 : (rows_e - t.m0 <= 64 ? 5 : 1)) : (narrow ? 2 : 0);
     } else if (pieces == 2) {
       t.n0 += piece * 128;
       t.kind = t.n0 < p.n ? 2 : -1;
@@ -1333,6 +1337,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
       else if (cur.kind == 2) gemm_tile<ELT, 4, 2>(p, smem, c, cur, next, pf);
       else if (cur.kind == 3) gemm_tile<ELT, 2, 2>(p, smem, c, cur, next, pf);
       else if (cur.kind == 4) gemm_tile<ELT, 1, 1>(p, smem, c, cur, next, pf);
+      else if (cur.kind == 5) gemm_tile<ELT, 1, 4>(p, smem, c, cur, next, pf);
     }
     cur = next;
   }
