@@ -608,6 +608,10 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
   // Fill instruction Q of the k-step at byte offset kbyte of every row, into ring slot SLOT (compile-time
   // slot: the LDS address is an immediate).  The k offset travels as the scalar offset: an instruction
   // immediate would also be added to the LDS address.
+  // The 64 x 64 pieces of a skinny tail read their weights once and from HBM (470 MB on the Mixtral shape, after
+  // the launch's other tiles): those fills are marked non-temporal, so that they do not push the output the launch
+  // has just written out of the Infinity Cache ahead of the kernel that reads it next.
+  constexpr int W_AUX = Ring<MB, NB>::tiny ? 2 : 0;  // cache policy of the weight fills: 2 = nt
   auto fill_one = [&](auto SLOT, auto Q, int kbyte) {
     constexpr int slot = decltype(SLOT)::value, q = decltype(Q)::value;
     if constexpr (q < XLOADS)
@@ -615,7 +619,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
                                                static_cast<int>(xoff[q]), kbyte, 0, 0);
     else
       __builtin_amdgcn_raw_ptr_buffer_load_lds(wrsrc, (lds_ptr_t)(wdst + slot * SB + (q - XLOADS) * 1024), 16,
-                                               static_cast<int>(woff[q - XLOADS]), kbyte, 0, 0);
+                                               static_cast<int>(woff[q - XLOADS]), kbyte, 0, W_AUX);
   };
   // The same fill as two instructions placed by hand: the LDS destination goes into M0 one MFMA slot ahead
   // of the load.  The builtin emits s_mov m0 / s_nop / buffer_load as one cluster; every instruction between
@@ -642,7 +646,8 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
     } else {
       const uint32_t vo = woff[q - XLOADS];
       __amdgpu_buffer_rsrc_t r = wrsrc;
-      asm volatile("buffer_load_dwordx4 %0, %1, %2 offen lds" : : "v"(vo), "s"(r), "s"(kbyte) : "memory");
+      if constexpr (W_AUX == 2) asm volatile("buffer_load_dwordx4 %0, %1, %2 offen nt lds" : : "v"(vo), "s"(r), "s"(kbyte) : "memory");
+      else asm volatile("buffer_load_dwordx4 %0, %1, %2 offen lds" : : "v"(vo), "s"(r), "s"(kbyte) : "memory");
     }
   };
   // Same with a run-time slot, for the last steps of a tile; a k-step past the end of K (the phantom
@@ -662,7 +667,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
                                                static_cast<int>(in ? xoff[q] : zoff), kbyte, 0, 0);
     else
       __builtin_amdgcn_raw_ptr_buffer_load_lds(in ? wrsrc : zrsrc, (lds_ptr_t)(wdst + slot * SB + (q - XLOADS) * 1024),
-                                               16, static_cast<int>(in ? woff[q - XLOADS] : zoff), kbyte, 0, 0);
+                                               16, static_cast<int>(in ? woff[q - XLOADS] : zoff), kbyte, 0, W_AUX);
   };
 
   typename Geom<ELT>::Acc acc[MBK][NBK];
