@@ -257,6 +257,11 @@ def aux_measurements(torch, capi, configs, a, wl, dev, gen, tensors):
         kernels["gemm_layer1_uniform_splits"] = gemm_entry(time_loop(torch, lambda: capi.grouped_gemm(y, w2, spu, out=z32, row_scale=row_w), 20), gemm_flops)
         kernels["gemm_layer0_workload_splits"] = gemm_entry(time_loop(torch, lambda: capi.grouped_gemm(x, w1, sp, out=y, gather_a=giu), 20), gemm_flops)
         kernels["gemm_layer1_workload_splits"] = gemm_entry(time_loop(torch, lambda: capi.grouped_gemm(y, w2, sp, out=z32, row_scale=row_w), 20), gemm_flops)
+        # the two forms of the MFMA kernel's ring fills, forced, on the workload's splits (the default rule runs layer0,
+        # whose rows are gathered, with half lines and layer1, K = 28 KiB per row, with whole lines)
+        for form, flag in (("half_line_fills", capi.SCHED_HALF_LINE_FILLS), ("whole_line_fills", capi.SCHED_WHOLE_LINE_FILLS)):
+            kernels[f"gemm_layer0_{form}"] = gemm_entry(time_loop(torch, lambda: capi.grouped_gemm(x, w1, sp, out=y, gather_a=giu, sched_flags=flag), 20), gemm_flops)
+            kernels[f"gemm_layer1_{form}"] = gemm_entry(time_loop(torch, lambda: capi.grouped_gemm(y, w2, sp, out=z32, row_scale=row_w, sched_flags=flag), 20), gemm_flops)
         del z32, spu
 
     # -- stand-alone HBM kernels --
@@ -333,6 +338,11 @@ def aux_measurements(torch, capi, configs, a, wl, dev, gen, tensors):
         # per-row x per-output-channel scales (and the top-8 weight folded into the row scale) in the epilogue
         t_f8 = time_loop(torch, lambda: capi.grouped_gemm(a8, b8, sp5, out=d5, row_scale=rs5, col_scale=cs5), 20)
         kernels[f"gemm_fp8_c5_{tag}"] = gemm_entry(t_f8, f5, PEAK_FP8_TFLOPS, "frac_fp8_peak")
+        # the same launch with whole-line ring fills forced (not the default at these K: uniform splits like these gain,
+        # ragged ones lose)
+        t_f8w = time_loop(torch, lambda: capi.grouped_gemm(a8, b8, sp5, out=d5, row_scale=rs5, col_scale=cs5,
+                                                           sched_flags=capi.SCHED_WHOLE_LINE_FILLS), 20)
+        kernels[f"gemm_fp8_c5_{tag}_whole_line_fills"] = gemm_entry(t_f8w, f5, PEAK_FP8_TFLOPS, "frac_fp8_peak")
         # 1 x 128 activation scales x 128 x 128 weight scales, promoted every 128 of K
         sa = torch.rand(m5 // 128, k5 // 128, 128, generator=gen, device=dev) + 0.5
         sb = torch.rand(e5, n5 // 128, k5 // 128, generator=gen, device=dev) + 0.5

@@ -162,10 +162,19 @@ SCHED_WHOLE_TAIL_TILES = 1
 SCHED_NO_HALF_TILES = 2
 SCHED_NO_SKINNY_TAIL = 4
 SCHED_FORCE_SKINNY_TAIL = 8
+SCHED_HALF_LINE_FILLS = 16
+SCHED_WHOLE_LINE_FILLS = 32
+
+
+# Form of the MFMA kernel's ring fills for calls that name none themselves: 0 (the library's rule by shape),
+# SCHED_HALF_LINE_FILLS or SCHED_WHOLE_LINE_FILLS.  Results are bit-identical either way.
+default_fill_form = 0
 
 
 def _gemm_args(a, b, splits, out, gather_a, scatter_d, alpha, row_scale, col_scale, scalar_scale, scalar_scale_dev,
                max_rows, out_dtype, cu_margin, raster_rows, sched_flags, need_out=True):
+    if not sched_flags & (SCHED_HALF_LINE_FILLS | SCHED_WHOLE_LINE_FILLS):
+        sched_flags |= default_fill_form
     dtype = _DTYPES.get(a.dtype)
     if dtype is None:
         raise ValueError(f"unsupported input dtype {a.dtype}")

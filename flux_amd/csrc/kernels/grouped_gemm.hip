@@ -196,8 +196,11 @@ int run_grouped_gemm(const fluxmi_grouped_gemm_args *args, int ngroups, const vo
                  "grouped_gemm: raster_rows=%d outside [0,1024]", args->raster_rows);
   FLUXMI_REQUIRE(args->cu_margin >= 0, FLUXMI_ERR_INVALID_ARG, "grouped_gemm: negative cu_margin");
   FLUXMI_REQUIRE((args->sched_flags & ~(FLUXMI_SCHED_WHOLE_TAIL_TILES | FLUXMI_SCHED_NO_HALF_TILES |
-                                        FLUXMI_SCHED_NO_SKINNY_TAIL | FLUXMI_SCHED_FORCE_SKINNY_TAIL)) == 0,
+                                        FLUXMI_SCHED_NO_SKINNY_TAIL | FLUXMI_SCHED_FORCE_SKINNY_TAIL | FLUXMI_SCHED_HALF_LINE_FILLS |
+                                        FLUXMI_SCHED_WHOLE_LINE_FILLS)) == 0,
                  FLUXMI_ERR_INVALID_ARG, "grouped_gemm: unknown sched_flags 0x%x", args->sched_flags);
+  FLUXMI_REQUIRE((args->sched_flags & FLUXMI_SCHED_HALF_LINE_FILLS) == 0 || (args->sched_flags & FLUXMI_SCHED_WHOLE_LINE_FILLS) == 0,
+                 FLUXMI_ERR_INVALID_ARG, "grouped_gemm: sched_flags ask for half-line and whole-line fills at once");
   // fp32 outputs beyond half a GB go out non-temporally (measured on a 805 MB intermediate: the GEMM 5 % faster,
   // the reduce that reads it unchanged; at 268 MB the GEMM is unchanged and the reduce 10 % slower).
   p.nt_stores = (args->d_fp32 != 0 && accumulate_rows == 0 && static_cast<int64_t>(args->max_rows) * args->n * 4 > (int64_t{512} << 20)) ? 1 : 0;
@@ -216,10 +219,20 @@ int run_grouped_gemm(const fluxmi_grouped_gemm_args *args, int ngroups, const vo
     const int64_t tiles_n = (args->n + BN - 1) / BN * ngroups;
     const int64_t max_tiles = (static_cast<int64_t>(args->max_rows) / BM + args->nexperts) * tiles_n;
     const int grid = static_cast<int>(max_tiles < cus ? max_tiles : cus);
+    // Form of the ring fills.  Whole 128-byte lines cost the memory pipeline less per byte and need one barrier per
+    // pair of k-steps, but a pair's 64 KiB stay in LDS for both of its steps, so fewer fills are in flight: faster
+    // (2-5 %) where the compute units that share operand panels run in step (uniform row counts) or K is long, slower
+    // (up to 7 %) on ragged row counts at short K, where single units run ahead of the others and every one of their
+    // fills misses L2.  Default: whole lines for rows of K of at least 16 KiB that are not gathered (measured on
+    // 8 ragged experts at K = 14336 bf16: -2.5 %), half lines otherwise; the flags force either, and `profiling()`
+    // of the layer ops times both on the caller's own row counts.
+    const int64_t kbytes = static_cast<int64_t>(args->k) * (args->dtype == FLUXMI_FP8_E4M3 ? 1 : 2);
+    const bool lines = (args->sched_flags & FLUXMI_SCHED_WHOLE_LINE_FILLS) != 0 ||
+                       ((args->sched_flags & FLUXMI_SCHED_HALF_LINE_FILLS) == 0 && args->gather_a == nullptr && kbytes >= 16384);
     const int rc = bs != nullptr ? launch_grouped_gemm_fp8_blockscale(p, grid, s)
-                   : args->dtype == FLUXMI_BF16 ? launch_grouped_gemm_bf16(p, grid, s)
-                   : args->dtype == FLUXMI_FP16 ? launch_grouped_gemm_f16(p, grid, s)
-                                                : launch_grouped_gemm_fp8(p, grid, s);
+                   : args->dtype == FLUXMI_BF16 ? (lines ? launch_grouped_gemm_bf16_lines(p, grid, s) : launch_grouped_gemm_bf16(p, grid, s))
+                   : args->dtype == FLUXMI_FP16 ? launch_grouped_gemm_f16(p, grid, s)  // the half-line form only
+                                                : (lines ? launch_grouped_gemm_fp8_lines(p, grid, s) : launch_grouped_gemm_fp8(p, grid, s));
     if (rc != FLUXMI_OK) return rc;
   } else {
     const int grid = cus * 8;

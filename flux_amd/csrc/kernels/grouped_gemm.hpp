@@ -100,5 +100,9 @@ int launch_grouped_gemm_bf16(const GemmParams &p, int grid, hipStream_t s);
 int launch_grouped_gemm_f16(const GemmParams &p, int grid, hipStream_t s);
 int launch_grouped_gemm_fp8(const GemmParams &p, int grid, hipStream_t s);
 int launch_grouped_gemm_fp8_blockscale(const GemmParams &p, int grid, hipStream_t s);
+// The bf16 and fp8 kernels with whole-line ring fills (FLUXMI_SCHED_WHOLE_LINE_FILLS and the default rule in
+// grouped_gemm.hip); fp16 has the half-line form only.
+int launch_grouped_gemm_bf16_lines(const GemmParams &p, int grid, hipStream_t s);
+int launch_grouped_gemm_fp8_lines(const GemmParams &p, int grid, hipStream_t s);
 
 }  // namespace fluxmi

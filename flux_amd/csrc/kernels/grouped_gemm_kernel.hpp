@@ -6,6 +6,10 @@
 namespace fluxmi {
 namespace {
 
+// The device code below is compiled in the device pass only; the host pass sees the kernel's declaration with an empty
+// body (all it needs for the launch stub).
+#if defined(__HIP_DEVICE_COMPILE__)
+
 #define FLUXMI_WAITCNT(vm, lgkm) \
   __builtin_amdgcn_s_waitcnt(((vm)&15) | (((vm) >> 4) << 14) | (7 << 4) | ((lgkm) << 8))
 
@@ -25,6 +29,15 @@ __device__ __forceinline__ void load_to_lds16(const uint8_t *src, uint8_t *lds_b
 constexpr bool kHalfIsF16 = true;
 #else
 constexpr bool kHalfIsF16 = false;
+#endif
+
+// Which form of ring fills whole, half-height, half-width and 64-row tiles use: 64-byte half lines, one k-step per ring
+// stage (gemm_tile), or, if the including translation unit defines FLUXMI_LINE_FILLS, whole 128-byte lines, a pair of
+// k-steps per ring unit (gemm_tile_lines).
+#ifdef FLUXMI_LINE_FILLS
+constexpr bool kLineFills = true;
+#else
+constexpr bool kLineFills = false;
 #endif
 
 // Two floats to the packed 16-bit output type (bf16: one v_cvt_pk_bf16_f32; fp16: two v_cvt_f16_f32 and a pack),
@@ -99,6 +112,12 @@ struct TileCtx {
   int wave, lane, wn, wm;
   int fill_row, fill_chunk;
   int frag_off[2];
+  // The same for whole-line fills (one instruction covers 8 rows x 128 bytes, i.e. a pair of k-steps): the row of
+  // the 8 this lane fetches, its byte offset inside the row's 128 bytes for fill instructions over even / odd
+  // 8-row blocks, and its fragment offsets inside a 32 KiB operand unit.
+  int lfill_row;
+  int lfill_byte[2];
+  int lfrag_off[2];
   int nk;           // k-steps of 64 bytes per row, a partial last one included
   int nkf;          // whole k-steps
   int tail_chunks;  // 16-byte chunks of the partial last k-step (0: K is a whole number of k-steps)
@@ -424,6 +443,7 @@ struct TileOperands {
   uint32_t xoff[XL], woff[WL];
 };
 
+
 // What a tile leaves behind for the next one when that is a whole macro tile: its operand addressing,
 // with k-steps 0..3 already requested into ring slots 0..3 ahead of the epilogue, so that their latency
 // passes while the epilogue runs.
@@ -552,13 +572,153 @@ __device__ __forceinline__ void issue_first_pairs(const TileOperands<XL, WL> &op
   }
 }
 
+// ---- the same tile with whole-line ring fills ---------------------------------------------------------------
+// The unit of the ring is one operand's share of a PAIR of k-steps: 64*MB (64*NB) rows x 128 bytes, at most 32 KiB,
+// one of five ring slots; X of pair P is unit 2P, W of pair P unit 2P + 1, unit u lies in slot u % 5.  A fill
+// instruction fetches 8 rows x 128 bytes, whole cache lines (the 64-byte form fetches the two halves of a line with
+// two instructions: the second finds the line in L1, but the memory pipeline handles it twice — measured on fills
+// alone 88 against 101 GB/s per compute unit).  During the even step of pair P the X unit of pair P + 2 is
+// requested (into the slot of W of pair P - 1), during the odd step its W unit (into the slot of X of pair P, whose
+// last fragment reads were issued during the even step).  A pair's units are read by both of its steps, so only odd
+// steps wait and synchronise: one `s_waitcnt vmcnt` and one barrier per pair of k-steps.  The look-ahead is what
+// the 64-byte ring has (a unit is requested two to three steps before its first read), the fills per step and the
+// LDS banks of the fragment reads are the same.
+template <int MB, int NB>
+struct LineRing {
+  static constexpr int XF = 2 * MB;  // fill instructions per wave and pair: X unit
+  static constexpr int WF = 2 * NB;  // ... W unit
+  static constexpr int UB = STAGE_BYTES;  // bytes of a ring slot
+  static constexpr int ROWB = 2 * KBYTES;  // bytes of a row in a unit
+};
+
+template <int XF, int WF>
+struct LineOperands {
+  __amdgpu_buffer_rsrc_t xrsrc, wrsrc;
+  uint32_t xoff[XF], woff[WF];
+};
+
+struct LinePrefetch {
+  bool valid;
+  LineOperands<8, 8> op;
+};
+
+template <int XF>
+__device__ __forceinline__ void load_gather_rows_lines(const GemmParams &p, const TileCtx &c, const TileDesc &t, int (&arow)[XF]) {
+#pragma unroll
+  for (int j = 0; j < XF; ++j) {
+    int xr = t.m0 + (XF * c.wave + j) * 8 + c.lfill_row;
+    if (xr > t.rows_e - 1) xr = t.rows_e - 1;
+    if (xr < 0) xr = 0;
+    arow[j] = p.gather_a[t.row_base + xr];
+  }
+}
+
+template <int XF, int WF>
+__device__ __forceinline__ void setup_operands_lines(const GemmParams &p, const TileCtx &c, const TileDesc &t,
+                                                     LineOperands<XF, WF> &op, const int *preloaded_rows = nullptr) {
+  const bool gathered = p.gather_a != nullptr;
+  const uint8_t *xbase = gathered ? p.a : p.a + static_cast<int64_t>(t.row_base + t.m0) * c.kbytes;
+  const int64_t xrows = gathered ? p.a_rows : t.rows_e - t.m0;
+  op.xrsrc = make_rsrc(xbase, xrows > 0 ? xrows * c.kbytes : 0xffffffffll);
+  int n0 = t.n0;
+  const int g = split_group(n0, p.n, p.ngroups);
+  op.wrsrc = make_rsrc(kernel_args()->b[g] + (static_cast<int64_t>(t.e) * p.n + n0) * c.kbytes, static_cast<int64_t>(p.n - n0) * c.kbytes);
+#pragma unroll
+  for (int j = 0; j < XF; ++j) {
+    int xr = t.m0 + (XF * c.wave + j) * 8 + c.lfill_row;
+    if (xr > t.rows_e - 1) xr = t.rows_e - 1;
+    int64_t arow = xr - t.m0;
+    if (gathered) {
+      arow = preloaded_rows ? preloaded_rows[j] : p.gather_a[t.row_base + xr];
+      if (p.a_rows > 0) arow = arow < 0 ? 0 : (arow >= p.a_rows ? p.a_rows - 1 : arow);
+    }
+    op.xoff[j] = static_cast<uint32_t>(arow * c.kbytes) + c.lfill_byte[j & 1];
+  }
+#pragma unroll
+  for (int j = 0; j < WF; ++j) {
+    int wr = n0 + (WF * c.wave + j) * 8 + c.lfill_row;
+    if (wr > p.n - 1) wr = p.n - 1;
+    op.woff[j] = static_cast<uint32_t>((wr - n0) * c.kbytes) + c.lfill_byte[j & 1];
+  }
+}
+
+// Fill instruction q of a unit (an operand's 128 bytes of K at byte offset kb of every row) into LDS at dst, whatever
+// kb is: a whole unit, the last unit of a K that is not a multiple of 128 bytes (lanes whose 16 bytes lie inside the
+// row fetch them, the others write zeros to their own LDS slot: an out-of-range direct-to-LDS load writes
+// nothing), or a unit past the end of K (requested from a page of zeros, so that the fill counts of the waits
+// hold).  `lane_byte` is the lane's byte offset inside the 128 bytes.
+__device__ __forceinline__ void fill_unit_any(__amdgpu_buffer_rsrc_t rsrc, uint32_t off, int lane_byte, int64_t kb, uint8_t *dst,
+                                              const TileCtx &c) {
+  if (kb + 128 <= c.kbytes) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)dst, 16, static_cast<int>(off), static_cast<int>(kb), 0, 0);
+  } else if (kb < c.kbytes) {  // wave-uniform
+    if (lane_byte < static_cast<int>(c.kbytes - kb)) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)dst, 16, static_cast<int>(off), static_cast<int>(kb), 0, 0);
+    } else {
+      *reinterpret_cast<u32x4 *>(dst + c.lane * 16) = u32x4{0u, 0u, 0u, 0u};
+    }
+    FLUXMI_WAITCNT(63, 0);
+  } else {
+    const __amdgpu_buffer_rsrc_t zrsrc = make_rsrc(g_zero_page, 1024);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(zrsrc, (lds_ptr_t)dst, 16, c.lane * 16, 0, 0, 0);
+  }
+}
+
+// Requests the first two pairs of a tile: units 0..3 (W0, X0, W1, X1) into ring slots 0..3.
+template <int XF, int WF>
+__device__ __forceinline__ void issue_first_units(const LineOperands<XF, WF> &op, uint8_t *smem, const TileCtx &c) {
+  constexpr int UB = STAGE_BYTES;
+  if (c.kbytes >= 256) {  // all four are whole units (every K of practical interest): no per-fill choices
+#pragma unroll
+    for (int pr = 0; pr < 2; ++pr) {
+#pragma unroll
+      for (int q = 0; q < WF; ++q)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(op.wrsrc, (lds_ptr_t)(smem + (2 * pr) * UB + (WF * c.wave + q) * 1024), 16,
+                                                 static_cast<int>(op.woff[q]), pr * 128, 0, 0);
+#pragma unroll
+      for (int q = 0; q < XF; ++q)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(op.xrsrc, (lds_ptr_t)(smem + (2 * pr + 1) * UB + (XF * c.wave + q) * 1024), 16,
+                                                 static_cast<int>(op.xoff[q]), pr * 128, 0, 0);
+    }
+    return;
+  }
+#pragma unroll
+  for (int pr = 0; pr < 2; ++pr) {
+#pragma unroll
+    for (int q = 0; q < WF; ++q)
+      fill_unit_any(op.wrsrc, op.woff[q], c.lfill_byte[q & 1], pr * 128, smem + (2 * pr) * UB + (WF * c.wave + q) * 1024, c);
+#pragma unroll
+    for (int q = 0; q < XF; ++q)
+      fill_unit_any(op.xrsrc, op.xoff[q], c.lfill_byte[q & 1], pr * 128, smem + (2 * pr + 1) * UB + (XF * c.wave + q) * 1024, c);
+  }
+}
+
+// Operand addressing and first fills of the whole macro tile `next`, in the form its tile function expects.
+__device__ __forceinline__ void prefetch_whole_tile(const GemmParams &p, uint8_t *smem, const TileCtx &c, const TileDesc &next,
+                                                    TilePrefetch &pf, const int *rows) {
+  setup_operands<4, 4>(p, c, next, pf.op, rows);
+  issue_first_pairs<4, 4>(pf.op, smem, c);
+  pf.valid = true;
+}
+__device__ __forceinline__ void prefetch_whole_tile(const GemmParams &p, uint8_t *smem, const TileCtx &c, const TileDesc &next,
+                                                    LinePrefetch &pf, const int *rows) {
+  setup_operands_lines<8, 8>(p, c, next, pf.op, rows);
+  issue_first_units<8, 8>(pf.op, smem, c);
+  pf.valid = true;
+}
+
 // One output tile of (64*MB) rows x (64*NB) columns at rows [m0, ..) of expert e, columns [n0, ..).
 // (MB, NB) = (4, 4) is the macro tile, (2, 4) its upper half (for the last rows of an expert); (4, 2) and
 // (2, 2) are the 256x128 and 128x128 pieces a tile of the last, partly filled round is cut into.  Waves
 // are laid out 2 x 2.
-template <int ELT, int MB, int NB>
+template <int ELT, int MB, int NB, class PF>
 __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, const TileCtx &c, const TileDesc &t,
-                                          const TileDesc &next, TilePrefetch &pf) {
+                                          const TileDesc &next, PF &pf) {
+  // PF = TilePrefetch: every tile shape of the launch runs this function.  PF = LinePrefetch: whole, half-height,
+  // half-width and 64-row tiles run gemm_tile_lines, and a whole tile that follows one of this function's tiles
+  // gets its first fills in that function's form.
+  constexpr bool LINES_NEXT = std::is_same<PF, LinePrefetch>::value;
+  static_assert(!LINES_NEXT || MB != 4 || NB != 4, "whole tiles of such a launch run gemm_tile_lines");
   constexpr int XLOADS = MB;           // direct-to-LDS instructions per wave per stage, X tile
   constexpr int WLOADS = NB;           // same, W tile
   constexpr int LOADS = XLOADS + WLOADS;
@@ -581,7 +741,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
   // Operand addressing: prepared by the previous tile together with the first fills, or set up here.
   bool prefetched = false;
   TileOperands<XLOADS, WLOADS> op;
-  if constexpr (MB == 4 && NB == 4) {
+  if constexpr (MB == 4 && NB == 4 && !LINES_NEXT) {
     if (pf.valid) {
       prefetched = true;
       op = pf.op;
@@ -590,9 +750,13 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
   if (!prefetched) setup_operands<XLOADS, WLOADS>(p, c, t, op);
   // The gather indices of the next tile (when it is a whole macro tile, whose first fills this tile requests
   // ahead of its epilogue): requested now, so that their latency passes under this tile's main loop.
-  int next_rows[4] = {0, 0, 0, 0};
+  constexpr int NPRE = LINES_NEXT ? 8 : 4;  // row indices per lane of a whole tile's X fills
+  int next_rows[NPRE] = {};
   const bool preload_next = next.kind == 0 && p.gather_a != nullptr;
-  if (preload_next) load_gather_rows<4>(p, c, next, next_rows);
+  if (preload_next) {
+    if constexpr (LINES_NEXT) load_gather_rows_lines<NPRE>(p, c, next, next_rows);
+    else load_gather_rows<NPRE>(p, c, next, next_rows);
+  }
   const __amdgpu_buffer_rsrc_t xrsrc = op.xrsrc, wrsrc = op.wrsrc;
   const __amdgpu_buffer_rsrc_t zrsrc = make_rsrc(g_zero_page, 1024);
   const uint32_t zoff = lane * 16;
@@ -823,11 +987,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
   // A whole macro tile next: its first four k-steps are requested now, into ring slots 0..3; the
   // epilogue's LDS windows lie in slot 4.
   pf.valid = false;
-  if (next.kind == 0) {
-    setup_operands<4, 4>(p, c, next, pf.op, preload_next ? next_rows : nullptr);
-    issue_first_pairs<4, 4>(pf.op, smem, c);
-    pf.valid = true;
-  }
+  if (next.kind == 0) prefetch_whole_tile(p, smem, c, next, pf, preload_next ? next_rows : nullptr);
   uint8_t *windows = smem + 4 * STAGE_BYTES + wave * 8192;  // one 8 KiB window per wave
   const int wrow0 = m0 + wm * (32 * MB);
   {
@@ -852,6 +1012,240 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
       }
     };
     store(acc);
+  }
+  __builtin_amdgcn_s_barrier();  // the LDS windows are free again before the next tile's fills start
+}
+
+template <int ELT, int MB, int NB>
+__device__ __forceinline__ void gemm_tile_lines(const GemmParams &p, uint8_t *smem, const TileCtx &c, const TileDesc &t,
+                                                const TileDesc &next, LinePrefetch &pf) {
+  constexpr int XF = LineRing<MB, NB>::XF, WF = LineRing<MB, NB>::WF;
+  constexpr int UB = LineRing<MB, NB>::UB, ROWB = LineRing<MB, NB>::ROWB;
+  constexpr int BLK = Geom<ELT>::BLK, NCH = Geom<ELT>::NCH;
+  constexpr int MBK = 32 * MB / BLK, NBK = 32 * NB / BLK;  // operand blocks of a wave
+  constexpr int NR = (MBK + NBK) * NCH;                    // fragment reads per k-step (16 bytes per lane each)
+  constexpr int NM = MBK * NBK;                            // MFMAs per k-step
+  constexpr int RSPAN = NM / 2;                            // MFMA slots over which the fragment reads of a step are spread
+  constexpr int TRIP = 10;                                 // k-steps after which ring slots and fragment sets repeat
+  const int wave = c.wave, wm = c.wm, wn = c.wn, nk = c.nk;
+  const int e = t.e, row_base = t.row_base, rows_e = t.rows_e, m0 = t.m0;
+
+  bool prefetched = false;
+  LineOperands<XF, WF> op;
+  if constexpr (MB == 4 && NB == 4) {
+    if (pf.valid) {
+      prefetched = true;
+      op = pf.op;
+    }
+  }
+  if (!prefetched) setup_operands_lines<XF, WF>(p, c, t, op);
+  int next_rows[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  const bool preload_next = next.kind == 0 && p.gather_a != nullptr;
+  if (preload_next) load_gather_rows_lines<8>(p, c, next, next_rows);
+  const __amdgpu_buffer_rsrc_t xrsrc = op.xrsrc, wrsrc = op.wrsrc;
+  uint32_t xoff[XF], woff[WF];
+#pragma unroll
+  for (int j = 0; j < XF; ++j) xoff[j] = op.xoff[j];
+#pragma unroll
+  for (int j = 0; j < WF; ++j) woff[j] = op.woff[j];
+  uint8_t *xdst = smem + (XF * wave) * 1024;  // this wave's first fill block inside an X unit
+  uint8_t *wdst = smem + (WF * wave) * 1024;
+  const uint32_t xdst32 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)xdst));
+  const uint32_t wdst32 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)wdst));
+
+  // Fill instruction Q of the X (IS_W: W) unit at byte offset kbyte of every row into ring slot SLOT, as one cluster
+  // (the builtin writes M0 itself) ...
+  auto fill_one = [&](auto IS_W, auto SLOT, auto Q, int kbyte) {
+    constexpr int slot = decltype(SLOT)::value, q = decltype(Q)::value;
+    if constexpr (!decltype(IS_W)::value)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(xrsrc, (lds_ptr_t)(xdst + slot * UB + q * 1024), 16, static_cast<int>(xoff[q]), kbyte, 0, 0);
+    else
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(wrsrc, (lds_ptr_t)(wdst + slot * UB + q * 1024), 16, static_cast<int>(woff[q]), kbyte, 0, 0);
+  };
+  // ... or as two instructions placed by hand: the LDS destination goes into M0 one MFMA slot ahead of the load.
+  // Nothing else in the k loop uses M0; the compiler is not told that M0 changes, which is safe while it puts no M0
+  // use of its own between the two (the schedule barriers around every MFMA slot see to that).
+  auto fill_m0 = [&](auto IS_W, auto SLOT, auto Q) {
+    constexpr int slot = decltype(SLOT)::value, q = decltype(Q)::value;
+    const uint32_t dst = (decltype(IS_W)::value ? wdst32 : xdst32) + slot * UB + q * 1024;
+    asm volatile("s_mov_b32 m0, %0" : : "s"(dst) : "memory");
+  };
+  auto fill_go = [&](auto IS_W, auto Q, int kbyte) {
+    constexpr int q = decltype(Q)::value;
+    if constexpr (decltype(IS_W)::value) {
+      const uint32_t vo = woff[q];
+      __amdgpu_buffer_rsrc_t r = wrsrc;
+      asm volatile("buffer_load_dwordx4 %0, %1, %2 offen lds" : : "v"(vo), "s"(r), "s"(kbyte) : "memory");
+    } else {
+      const uint32_t vo = xoff[q];
+      __amdgpu_buffer_rsrc_t r = xrsrc;
+      asm volatile("buffer_load_dwordx4 %0, %1, %2 offen lds" : : "v"(vo), "s"(r), "s"(kbyte) : "memory");
+    }
+  };
+
+  typename Geom<ELT>::Acc acc[MBK][NBK];
+#pragma unroll
+  for (int i = 0; i < MBK; ++i)
+#pragma unroll
+    for (int j = 0; j < NBK; ++j)
+#pragma unroll
+      for (int v = 0; v < Geom<ELT>::NACC; ++v) acc[i][j][v] = 0.f;
+
+  // Fragment addresses: per lane and 16-byte chunk s a base for each operand; slot, block and k-step parity add a
+  // compile-time offset.  LDS instructions carry 16 bits of offset, so three bases 64 KiB apart.
+  const uint8_t *xfrag[3][NCH], *wfrag[3][NCH];
+#pragma unroll
+  for (int hi = 0; hi < 3; ++hi)
+#pragma unroll
+    for (int s = 0; s < NCH; ++s) {
+      xfrag[hi][s] = smem + hi * 65536 + wm * (32 * MB) * ROWB + c.lfrag_off[s];
+      wfrag[hi][s] = smem + hi * 65536 + wn * (32 * NB) * ROWB + c.lfrag_off[s];
+    }
+  i32x4 xa[MBK][NCH], wa[NBK][NCH], xb[MBK][NCH], wb[NBK][NCH];
+  // Fragment read R of k-step U (counted within a trip; step u is half u & 1 of pair u >> 1).
+  auto read_one = [&](auto U, auto R, i32x4 (&xf)[MBK][NCH], i32x4 (&wf)[NBK][NCH]) {
+    constexpr int u = decltype(U)::value % TRIP, r = decltype(R)::value;
+    constexpr int ws = (2 * (u >> 1)) % 5, xs = (2 * (u >> 1) + 1) % 5, h = u & 1;
+    constexpr int s = r / (MBK + NBK), q = r % (MBK + NBK);
+    if constexpr (q < NBK)
+      wf[q][s] = *reinterpret_cast<const i32x4 *>(wfrag[(ws * UB) / 65536][s] + (ws * UB) % 65536 + q * BLK * ROWB + h * 512);
+    else
+      xf[q - NBK][s] = *reinterpret_cast<const i32x4 *>(xfrag[(xs * UB) / 65536][s] + (xs * UB) % 65536 + (q - NBK) * BLK * ROWB + h * 512);
+  };
+  // One k-step, number U of a trip of ten: MFMAs on `cur`, the fragments of step U + 1 into `nxt`, and the fills of
+  // one unit of pair U / 2 + 2 (even: X, odd: W), one fill per MFMA slot at most when there are slots enough.
+  // GUARDED (the last steps of a tile, which run the same code with the same ring slots: they start at a multiple
+  // of ten): the unit may be the last one of a K that is not a multiple of 128 bytes, or lie past the end of K.  Its
+  // fills then go through flat addresses, per lane either its 16 bytes of the operand or, where those lie past the
+  // end of the row, 16 bytes of a page of zeros; one vector-memory instruction per fill either way, so the fill
+  // counts of the waits hold.  kb is the byte offset along K of step 0 of the trip; xbase / wbase (guarded steps
+  // only) are the operands' first bytes.
+  auto step = [&](auto GUARDED, auto U, int64_t kb, const uint8_t *xbase, const uint8_t *wbase, i32x4 (&xc)[MBK][NCH],
+                  i32x4 (&wc)[NBK][NCH], i32x4 (&xn)[MBK][NCH], i32x4 (&wn_)[NBK][NCH]) {
+    constexpr bool guarded = decltype(GUARDED)::value;
+    constexpr int u = decltype(U)::value;
+    constexpr bool even = (u & 1) == 0;
+    constexpr int pr2 = (u >> 1) + 2;                      // pair whose unit this step requests
+    constexpr int fslot = (2 * pr2 + (even ? 0 : 1)) % 5;  // ring slot of that unit
+    constexpr int NF = even ? WF : XF;
+    constexpr bool SPLIT = !guarded && NF < NM;  // every fill has an MFMA slot of its own, and the slot before it for its M0 write
+    static_assert(!SPLIT || (NF - 1) * NM / NF + 1 < NM, "the last fill's load still lies inside the step");
+    typedef std::integral_constant<bool, even> IsW;
+    const int kbyte = static_cast<int>(kb) + pr2 * 128;
+    int valid = 128;                 // guarded: bytes of the unit's 128 that lie inside K
+    const uint8_t *gbase = nullptr;  // ... and the operand's first byte of the unit
+    if constexpr (guarded) {
+      const int64_t rem = c.kbytes - (kb + pr2 * 128);
+      valid = rem >= 128 ? 128 : (rem <= 0 ? 0 : static_cast<int>(rem));
+      gbase = (even ? wbase : xbase) + (rem > 0 ? kb + pr2 * 128 : 0);
+    }
+    if constexpr (!even) {
+      FLUXMI_WAITCNT(WF, 15);        // everything but the W unit requested during the even step has landed: pair u/2 + 1
+      __builtin_amdgcn_s_barrier();  // ... for every wave's share; and everybody is done reading W of this pair
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<0, NM>([&](auto T) {
+      constexpr int t = decltype(T)::value;
+      static_for<0, NR>([&](auto R) {
+        constexpr int r = decltype(R)::value;
+        if constexpr (r * RSPAN / NR == t) read_one(std::integral_constant<int, u + 1>{}, R, xn, wn_);
+      });
+      static_for<0, NF>([&](auto Q) {
+        constexpr int q = decltype(Q)::value;
+        if constexpr (guarded) {
+          if constexpr (q * NM / NF == t) {
+            uint32_t off;
+            if constexpr (even) off = woff[q];
+            else off = xoff[q];
+            const uint8_t *src = c.lfill_byte[q & 1] < valid ? gbase + off : g_zero_page + c.lane * 16;
+            __builtin_amdgcn_global_load_lds((gbl_ptr_t)src, (lds_ptr_t)((even ? wdst : xdst) + fslot * UB + q * 1024), 16, 0, 0);
+          }
+        } else if constexpr (SPLIT) {
+          if constexpr (q * NM / NF + 1 == t) fill_go(IsW{}, Q, kbyte);
+        } else {
+          if constexpr (q * NM / NF == t) fill_one(IsW{}, std::integral_constant<int, fslot>{}, Q, kbyte);
+        }
+      });
+      static_for<0, NF>([&](auto Q) {
+        constexpr int q = decltype(Q)::value;
+        if constexpr (SPLIT && q * NM / NF == t) fill_m0(IsW{}, std::integral_constant<int, fslot>{}, Q);
+      });
+      mfma_slot<ELT, MBK, NBK>(t, xc, wc, acc);
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    FLUXMI_WAITCNT(63, 0);  // the fragments of the next step are in registers (requested long ago)
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  // ---- prologue: the first two pairs are requested here or by the previous tile ahead of its epilogue ----------
+  FLUXMI_WAITCNT(0, 0);  // stores of the previous tile's epilogue (and, if it requested them, the first fills)
+  if (!prefetched) issue_first_units<XF, WF>(op, smem, c);
+  FLUXMI_WAITCNT(XF + WF, 15);  // pair 0 has landed
+  __builtin_amdgcn_s_barrier();
+  static_for<0, NR>([&](auto R) { read_one(std::integral_constant<int, 0>{}, R, xa, wa); });
+  FLUXMI_WAITCNT(63, 0);
+
+  // ---- main loop: whole trips while every unit a trip requests (up to pair 5 * trip + 6) is a whole one, then the
+  // remaining 4 .. 13 steps pair by pair with guarded fills; an odd number of k-steps ends with a step on zeros -----
+  const int nkf = c.nkf;
+  const int nfast = nkf >= TRIP + 4 ? (nkf - (TRIP + 4)) / TRIP + 1 : 0;
+  int kbase = 0;
+  for (int trip = 0; trip < nfast; ++trip) {
+    static_for<0, TRIP / 2>([&](auto H) {
+      constexpr int u = 2 * decltype(H)::value;
+      step(std::false_type{}, std::integral_constant<int, u>{}, kbase, nullptr, nullptr, xa, wa, xb, wb);
+      step(std::false_type{}, std::integral_constant<int, u + 1>{}, kbase, nullptr, nullptr, xb, wb, xa, wa);
+    });
+    kbase += TRIP * KBYTES;
+  }
+  if (TRIP * nfast < nk) {
+    const KernArgs pe = kernel_args();
+    const uint8_t *xbase = pe->gather_a != nullptr ? pe->a : pe->a + static_cast<int64_t>(row_base + m0) * c.kbytes;
+    int n0g = t.n0;
+    const int gg = split_group(n0g, pe->n, pe->ngroups);
+    const uint8_t *wbase = pe->b[gg] + (static_cast<int64_t>(e) * pe->n + n0g) * c.kbytes;
+    int64_t kb = static_cast<int64_t>(kbase);
+    for (int ks = TRIP * nfast; ks < nk; ks += TRIP, kb += TRIP * KBYTES) {
+      static_for<0, TRIP / 2>([&](auto H) {
+        constexpr int u = 2 * decltype(H)::value;
+        if (ks + u < nk) {
+          step(std::true_type{}, std::integral_constant<int, u>{}, kb, xbase, wbase, xa, wa, xb, wb);
+          step(std::true_type{}, std::integral_constant<int, u + 1>{}, kb, xbase, wbase, xb, wb, xa, wa);
+        }
+      });
+    }
+  }
+
+  // ---- epilogue ---------------------------------------------------------------------------------
+  FLUXMI_WAITCNT(0, 0);          // this wave's trailing ring fills have landed
+  __builtin_amdgcn_s_barrier();  // ... and everybody else's; nobody reads the ring any more
+  pf.valid = false;
+  if (next.kind == 0) {
+    setup_operands_lines(p, c, next, pf.op, preload_next ? next_rows : nullptr);
+    issue_first_units(pf.op, smem, c);
+    pf.valid = true;
+  }
+  uint8_t *windows = smem + 4 * STAGE_BYTES + wave * 8192;  // one 8 KiB window per wave, in ring slot 4
+  const int wrow0 = m0 + wm * (32 * MB);
+  {
+    const KernArgs pe = kernel_args();
+    int n0 = t.n0;
+    const int g = split_group(n0, pe->n, pe->ngroups);
+    const int wcol0 = n0 + wn * (32 * NB);
+    const bool full = wrow0 + 32 * MB <= rows_e && wcol0 + 32 * NB <= pe->n && pe->scatter_d == nullptr &&
+                      pe->accumulate == 0;
+    const bool out_f32 = pe->d_fp32 != 0;
+    const bool scaled = !(c.scalar == 1.f && pe->alpha[g] == nullptr && pe->row_scale == nullptr && pe->col_scale == nullptr);
+    if (full && !scaled) {
+      if (out_f32) store_tile<ELT, MB, NB, true, true, false>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, acc);
+      else store_tile<ELT, MB, NB, true, false, false>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, acc);
+    } else if (full) {
+      if (out_f32) store_tile<ELT, MB, NB, true, true, true>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, acc);
+      else store_tile<ELT, MB, NB, true, false, true>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, acc);
+    } else {
+      if (out_f32) store_tile<ELT, MB, NB, false, true, true>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, acc);
+      else store_tile<ELT, MB, NB, false, false, true>(windows, c, g, e, row_base, rows_e, wrow0, wcol0, acc);
+    }
   }
   __builtin_amdgcn_s_barrier();  // the LDS windows are free again before the next tile's fills start
 }
@@ -1126,8 +1520,11 @@ __device__ __forceinline__ void gemm_tile_blockscaled(const GemmParams &p, uint8
   __builtin_amdgcn_s_barrier();  // the LDS windows are free again before the next tile's fills start
 }
 
+#endif  // __HIP_DEVICE_COMPILE__
+
 template <int ELT, bool BS = false>
 __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];  // STAGES x (X tile | W tile)
 
   TileCtx c;
@@ -1167,6 +1564,27 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
       const int ch = 2 * (lane >> 5) + s;
       const int slot = ((lane & 3) << 2) | (ch ^ ((lane >> 2) & 3));
       c.frag_off[s] = ((lane & 31) >> 2) * 256 + slot * 16;
+    }
+  }
+  // Whole-line fills: a 1 KiB block of LDS holds 8 rows x 128 bytes as two halves of 512 bytes (k-step parity),
+  // each half laid out like 8 rows of the 64-byte layout above; lanes 0..31 of a fill instruction fetch the first
+  // 64 bytes of the 8 rows, lanes 32..63 the second (the memory pipeline still sees whole 128-byte lines), and the
+  // bank a fragment read touches is the same as in the 64-byte layout.
+  c.lfill_row = (lane & 31) >> 2;
+  if (ELT == 2) {
+    c.lfill_byte[0] = c.lfill_byte[1] = (lane >> 5) * 64 + (((lane & 3) ^ ((lane >> 3) & 3)) << 4);
+    const int r = lane & 15, ch = lane >> 4;
+    c.lfrag_off[0] = (r >> 3) * 1024 + (r & 7) * 64 + ((ch ^ ((r >> 1) & 3)) << 4);
+    c.lfrag_off[1] = 0;
+  } else {
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+      c.lfill_byte[b] = (lane >> 5) * 64 + (((lane & 3) ^ (((c.lfill_row >> 2) & 1) | (b << 1))) << 4);
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      const int r = lane & 31, ch = 2 * (lane >> 5) + s;
+      const int slot = ((lane & 3) << 2) | (ch ^ ((lane >> 2) & 3));
+      c.lfrag_off[s] = (r >> 3) * 1024 + ((r >> 2) & 1) * 256 + slot * 16;
     }
   }
   c.scalar = p.scalar;
@@ -1327,7 +1745,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
     return t;
   };
 
-  TilePrefetch pf;
+  typename std::conditional<kLineFills, LinePrefetch, TilePrefetch>::type pf;
   pf.valid = false;
   int item = virt;
   TileDesc cur = locate(item);
@@ -1336,6 +1754,13 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
     const TileDesc next = locate(item);
     if constexpr (BS) {
       if (cur.kind == 2) gemm_tile_blockscaled(p, smem, c, cur);
+    } else if constexpr (kLineFills) {
+      if (cur.kind == 0) gemm_tile_lines<ELT, 4, 4>(p, smem, c, cur, next, pf);
+      else if (cur.kind == 1) gemm_tile_lines<ELT, 2, 4>(p, smem, c, cur, next, pf);
+      else if (cur.kind == 2) gemm_tile_lines<ELT, 4, 2>(p, smem, c, cur, next, pf);
+      else if (cur.kind == 3) gemm_tile<ELT, 2, 2>(p, smem, c, cur, next, pf);
+      else if (cur.kind == 4) gemm_tile<ELT, 1, 1>(p, smem, c, cur, next, pf);
+      else if (cur.kind == 5) gemm_tile_lines<ELT, 1, 4>(p, smem, c, cur, next, pf);
     } else {
       if (cur.kind == 0) gemm_tile<ELT, 4, 4>(p, smem, c, cur, next, pf);
       else if (cur.kind == 1) gemm_tile<ELT, 2, 4>(p, smem, c, cur, next, pf);
@@ -1346,6 +1771,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
     }
     cur = next;
   }
+#endif  // __HIP_DEVICE_COMPILE__
 }
 
 template <int ELT, bool BS = false>

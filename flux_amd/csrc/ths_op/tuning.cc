@@ -36,6 +36,9 @@ std::vector<GemmLaunchTuning> gemm_tuning_candidates() {
   // where the few last rows of an expert run: as 64 x 64 pieces behind all other tiles, or in place
   out.push_back(GemmLaunchTuning{8, FLUXMI_SCHED_NO_SKINNY_TAIL});
   out.push_back(GemmLaunchTuning{8, FLUXMI_SCHED_FORCE_SKINNY_TAIL});
+  // both forms of the ring fills, whatever the default picks for the shape
+  out.push_back(GemmLaunchTuning{8, FLUXMI_SCHED_HALF_LINE_FILLS});
+  out.push_back(GemmLaunchTuning{8, FLUXMI_SCHED_WHOLE_LINE_FILLS});
   return out;
 }
 
@@ -128,7 +131,7 @@ size_t TuningTable::load_text(const std::string &text) {
     }
     if (seen != 255) fail("missing fields");
     if (t.raster_rows > 1024 || (t.sched_flags & ~(FLUXMI_SCHED_WHOLE_TAIL_TILES | FLUXMI_SCHED_NO_HALF_TILES | FLUXMI_SCHED_NO_SKINNY_TAIL |
-                                                  FLUXMI_SCHED_FORCE_SKINNY_TAIL)))
+                                                  FLUXMI_SCHED_FORCE_SKINNY_TAIL | FLUXMI_SCHED_HALF_LINE_FILLS | FLUXMI_SCHED_WHOLE_LINE_FILLS)))
       fail("raster_rows / sched_flags out of range");
     add(key, t);
     ++count;

@@ -147,6 +147,8 @@ typedef struct fluxmi_grouped_gemm_args {
 #define FLUXMI_SCHED_NO_HALF_TILES 2    /* run the last row tile of an expert 256 rows high even if 128 cover it, and the last column tile 256 wide even if 128 cover it */
 #define FLUXMI_SCHED_NO_SKINNY_TAIL 4    /* never move the last row tiles of experts that hold at most 64 rows behind all other tiles as 64 x 64 pieces */
 #define FLUXMI_SCHED_FORCE_SKINNY_TAIL 8 /* always do so (by default only when those pieces fill at most two rounds of the launch and K spans at least 128 steps of 64 bytes) */
+#define FLUXMI_SCHED_HALF_LINE_FILLS 16  /* fill the operand ring of the MFMA kernel with 64-byte half lines, one k-step per ring stage */
+#define FLUXMI_SCHED_WHOLE_LINE_FILLS 32 /* fill it with whole 128-byte lines, two k-steps per ring unit (default: only for rows of K of at least 16 KiB that are not gathered; fp16 operands always run the half-line form); not both flags */
 
 size_t fluxmi_grouped_gemm_workspace_bytes(const fluxmi_grouped_gemm_args *args);
 int fluxmi_grouped_gemm(const fluxmi_grouped_gemm_args *args, void *workspace,

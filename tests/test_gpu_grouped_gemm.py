@@ -11,6 +11,15 @@ RTOL, ATOL = 1e-2, 1e-2
 FP8_FROB = 3e-2
 
 
+
+@pytest.fixture(autouse=True, params=["half_line_fills", "whole_line_fills"])
+def fill_form(request):
+    """Every test of this module runs with both forms of the MFMA kernel's ring fills."""
+    from flux_amd import capi
+    capi.default_fill_form = capi.SCHED_HALF_LINE_FILLS if request.param == "half_line_fills" else capi.SCHED_WHOLE_LINE_FILLS
+    yield request.param
+    capi.default_fill_form = 0
+
 def assert_close(got_bf16, ref_f32, what=""):
     got = got_bf16.float().cpu()
     bad = (got - ref_f32).abs() > ATOL + RTOL * ref_f32.abs()
@@ -511,3 +520,33 @@ def test_skinny_tail_pieces_same_bits_as_in_place(dtype, ksteps):
     outs8 = capi.grouped_gemm_multi(a2, [w.cuda(), w2], sp, sched_flags=8)
     for o4, o8 in zip(outs4, outs8):
         assert torch.equal(o4, o8)
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp8"])
+@pytest.mark.parametrize("k", [128, 1024, 1040, 4096])
+def test_both_fill_forms_give_the_same_bits(dtype, k):
+    """Half-line and whole-line ring fills walk K in the same order with the same MFMAs: ragged experts (whole,
+    128-row, 64-row and partly filled tiles, pieces of the last round), a gather, a K with a partial last 128 bytes."""
+    from flux_amd import capi
+    rng = np.random.default_rng(k)
+    rows = [300, 0, 257, 64, 1000, 129, 513, 40]
+    m, n, tokens = sum(rows), 640, 700
+    sp = torch.tensor(rows, dtype=torch.int32).cuda()
+    gi = torch.from_numpy(rng.integers(0, tokens, m).astype(np.int32)).cuda()
+    if dtype == "bf16":
+        x = torch.from_numpy(rng.standard_normal((tokens, k), dtype=np.float32)).to(torch.bfloat16).cuda()
+        w = torch.from_numpy(rng.standard_normal((len(rows), n, k), dtype=np.float32) * 0.05).to(torch.bfloat16).cuda()
+    else:
+        x = torch.from_numpy(rng.standard_normal((tokens, k), dtype=np.float32)).to(torch.float8_e4m3fn).cuda()
+        w = torch.from_numpy(rng.standard_normal((len(rows), n, k), dtype=np.float32)).to(torch.float8_e4m3fn).cuda()
+    for kw in (dict(gather_a=gi), dict(gather_a=gi, out_dtype=torch.float32)):
+        half, kind = capi.grouped_gemm(x, w, sp, sched_flags=capi.SCHED_HALF_LINE_FILLS, want_kind=True, **kw)
+        whole = capi.grouped_gemm(x, w, sp, sched_flags=capi.SCHED_WHOLE_LINE_FILLS, **kw)
+        assert kind == 1
+        assert torch.equal(half, whole), f"{dtype} k={k} {list(kw)}: the two fill forms differ"
+    plain = x[gi.long()].contiguous()
+    half = capi.grouped_gemm(plain, w, sp, sched_flags=capi.SCHED_HALF_LINE_FILLS)
+    whole = capi.grouped_gemm(plain, w, sp, sched_flags=capi.SCHED_WHOLE_LINE_FILLS)
+    assert torch.equal(half, whole)
+    with pytest.raises(RuntimeError, match="at once"):
+        capi.grouped_gemm(plain, w, sp, sched_flags=capi.SCHED_HALF_LINE_FILLS | capi.SCHED_WHOLE_LINE_FILLS)

@@ -135,6 +135,11 @@ def test_tuning_text_round_trip_and_errors():
                               "sched_flags=8 reduce=fused\n"
                               "fluxmi_gemm_tuning dtype=bf16 experts=8 n=4096 k=14336 rows=16384 groups=1 raster_rows=8 "
                               "sched_flags=4 reduce=twopass\n") == 2
+    # ... and so is the form of the MFMA kernel's ring fills (16 half lines, 32 whole lines)
+    assert m.load_tuning_text("fluxmi_gemm_tuning dtype=e4m3 experts=32 n=2048 k=7168 rows=32768 groups=1 raster_rows=8 "
+                              "sched_flags=32\n"
+                              "fluxmi_gemm_tuning dtype=bf16 experts=8 n=4096 k=14336 rows=16384 groups=1 raster_rows=8 "
+                              "sched_flags=16\n") == 2
     with pytest.raises(RuntimeError, match="unknown reduce form"):
         m.load_tuning_text("fluxmi_gemm_tuning dtype=bf16 experts=1 n=1 k=1 rows=1 groups=1 raster_rows=1 sched_flags=0 reduce=maybe")
     m.clear_tuning_records()
