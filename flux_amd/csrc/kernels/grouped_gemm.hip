@@ -223,8 +223,9 @@ int run_grouped_gemm(const fluxmi_grouped_gemm_args *args, int ngroups, const vo
     // pair of k-steps, but a pair's 64 KiB stay in LDS for both of its steps, so fewer fills are in flight: faster
     // (2-5 %) where the compute units that share operand panels run in step (uniform row counts) or K is long, slower
     // (up to 7 %) on ragged row counts at short K, where single units run ahead of the others and every one of their
-    // fills misses L2.  Default: whole lines for rows of K of at least 16 KiB that are not gathered (measured on
-    // 8 ragged experts at K = 14336 bf16: -2.5 %), half lines otherwise; the flags force either, and `profiling()`
+    // fills misses L2.  Default: whole lines for rows that are not gathered and hold at least 16 KiB of K (measured on
+    // 8 ragged experts at K = 14336 bf16: -1.2 ... -2.5 %), half lines otherwise (a single-expert rule was tried: the
+    // dense bf16 GEMM 4096 x 12288 x 6144 gains under 1 %, the dense fp8 GEMMs 32768 x 7168 x 2048 lose 3-6 %); the flags force either, and `profiling()`
     // of the layer ops times both on the caller's own row counts.
     const int64_t kbytes = static_cast<int64_t>(args->k) * (args->dtype == FLUXMI_FP8_E4M3 ? 1 : 2);
     const bool lines = (args->sched_flags & FLUXMI_SCHED_WHOLE_LINE_FILLS) != 0 ||

@@ -6,6 +6,15 @@
 namespace fluxmi {
 namespace {
 
+// Which form of ring fills whole, half-height, half-width and 64-row tiles use: 64-byte half lines, one k-step per ring
+// stage (gemm_tile), or, if the including translation unit defines FLUXMI_LINE_FILLS, whole 128-byte lines, a pair of
+// k-steps per ring unit (gemm_tile_lines).
+#ifdef FLUXMI_LINE_FILLS
+constexpr bool kLineFills = true;
+#else
+constexpr bool kLineFills = false;
+#endif
+
 // The device code below is compiled in the device pass only; the host pass sees the kernel's declaration with an empty
 // body (all it needs for the launch stub).
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -29,15 +38,6 @@ __device__ __forceinline__ void load_to_lds16(const uint8_t *src, uint8_t *lds_b
 constexpr bool kHalfIsF16 = true;
 #else
 constexpr bool kHalfIsF16 = false;
-#endif
-
-// Which form of ring fills whole, half-height, half-width and 64-row tiles use: 64-byte half lines, one k-step per ring
-// stage (gemm_tile), or, if the including translation unit defines FLUXMI_LINE_FILLS, whole 128-byte lines, a pair of
-// k-steps per ring unit (gemm_tile_lines).
-#ifdef FLUXMI_LINE_FILLS
-constexpr bool kLineFills = true;
-#else
-constexpr bool kLineFills = false;
 #endif
 
 // Two floats to the packed 16-bit output type (bf16: one v_cvt_pk_bf16_f32; fp16: two v_cvt_f16_f32 and a pack),
@@ -1522,7 +1522,8 @@ __device__ __forceinline__ void gemm_tile_blockscaled(const GemmParams &p, uint8
 
 #endif  // __HIP_DEVICE_COMPILE__
 
-template <int ELT, bool BS = false>
+// LINE_FILLS is part of the kernel's name only (kLineFills decides the code): traces tell the two forms apart.
+template <int ELT, bool BS = false, bool LINE_FILLS = kLineFills>
 __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];  // STAGES x (X tile | W tile)
@@ -1777,9 +1778,9 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_mfma_kernel(const GemmP
 template <int ELT, bool BS = false>
 int launch_mfma(const GemmParams &p, int grid, hipStream_t s) {
   static std::atomic<uint64_t> lds_done{0};
-  const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(grouped_gemm_mfma_kernel<ELT, BS>), LDS_BYTES, lds_done);
+  const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(grouped_gemm_mfma_kernel<ELT, BS, kLineFills>), LDS_BYTES, lds_done);
   if (rc != FLUXMI_OK) return rc;
-  hipLaunchKernelGGL((grouped_gemm_mfma_kernel<ELT, BS>), dim3(grid), dim3(NTHREADS), LDS_BYTES, s, p);
+  hipLaunchKernelGGL((grouped_gemm_mfma_kernel<ELT, BS, kLineFills>), dim3(grid), dim3(NTHREADS), LDS_BYTES, s, p);
   return FLUXMI_OK;
 }
 
