@@ -573,16 +573,19 @@ __device__ __forceinline__ void issue_first_pairs(const TileOperands<XL, WL> &op
 }
 
 // ---- the same tile with whole-line ring fills ---------------------------------------------------------------
-// The unit of the ring is one operand's share of a PAIR of k-steps: 64*MB (64*NB) rows x 128 bytes, at most 32 KiB,
-// one of five ring slots; X of pair P is unit 2P, W of pair P unit 2P + 1, unit u lies in slot u % 5.  A fill
+// The unit of the ring is one operand's share of a PAIR of k-steps: 64*NB (64*MB) rows x 128 bytes, at most 32 KiB,
+// one of five ring slots; W of pair P is unit 2P, X of pair P unit 2P + 1, unit u lies in slot u % 5.  A fill
 // instruction fetches 8 rows x 128 bytes, whole cache lines (the 64-byte form fetches the two halves of a line with
 // two instructions: the second finds the line in L1, but the memory pipeline handles it twice — measured on fills
-// alone 88 against 101 GB/s per compute unit).  During the even step of pair P the X unit of pair P + 2 is
-// requested (into the slot of W of pair P - 1), during the odd step its W unit (into the slot of X of pair P, whose
-// last fragment reads were issued during the even step).  A pair's units are read by both of its steps, so only odd
-// steps wait and synchronise: one `s_waitcnt vmcnt` and one barrier per pair of k-steps.  The look-ahead is what
-// the 64-byte ring has (a unit is requested two to three steps before its first read), the fills per step and the
-// LDS banks of the fragment reads are the same.
+// alone 88 against 101 GB/s per compute unit).  During the even step of pair P the W unit of pair P + 2 is
+// requested (into the slot X of pair P - 1 has left), during the odd step its X unit (into the slot of W of pair P,
+// whose last fragment reads were issued during the even step).  A pair's units are read by both of its steps, so
+// only odd steps wait and synchronise: one `s_waitcnt vmcnt` and one barrier per pair of k-steps.  A unit is requested
+// two (X) to three (W) steps before its first read; the fills per step and the LDS banks of the fragment reads are
+// those of the 64-byte ring.  What the form costs: a pair's 64 KiB stay in LDS for both of its steps, so between 32
+// and 96 KiB of fills are in flight where the 64-byte ring keeps 64 to 96 — enough while the compute units that share
+// operand panels run in step and share each L2 miss, too little for a unit that runs apart from the others (ragged
+// row counts), which is why a launch picks its form by shape (grouped_gemm.hip).
 template <int MB, int NB>
 struct LineRing {
   static constexpr int XF = 2 * MB;  // fill instructions per wave and pair: X unit
