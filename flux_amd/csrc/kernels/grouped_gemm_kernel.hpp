@@ -761,8 +761,6 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
     else load_gather_rows<NPRE>(p, c, next, next_rows);
   }
   const __amdgpu_buffer_rsrc_t xrsrc = op.xrsrc, wrsrc = op.wrsrc;
-  const __amdgpu_buffer_rsrc_t zrsrc = make_rsrc(g_zero_page, 1024);
-  const uint32_t zoff = lane * 16;
   uint32_t xoff[XLOADS], woff[WLOADS];
 #pragma unroll
   for (int j = 0; j < XLOADS; ++j) xoff[j] = op.xoff[j];
@@ -817,26 +815,6 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
       else asm volatile("buffer_load_dwordx4 %0, %1, %2 offen lds" : : "v"(vo), "s"(r), "s"(kbyte) : "memory");
     }
   };
-  // Same with a run-time slot, for the last steps of a tile; a k-step past the end of K (the phantom
-  // second half of the last pair of an odd K) is filled from the zero page.
-  const int nkf = c.nkf;
-  auto fill_dyn = [&](int slot, auto Q, int kstep) {
-    constexpr int q = decltype(Q)::value;
-    const bool in = kstep < nkf;
-    const int kbyte = in ? kstep * KBYTES : 0;
-    if (kstep == nkf && c.tail_chunks != 0) {  // the partial last k-step (wave-uniform branch)
-      if constexpr (q < XLOADS) fill_partial(xrsrc, xoff[q], kstep * KBYTES, xdst + slot * SB + q * 1024, c);
-      else fill_partial(wrsrc, woff[q - XLOADS], kstep * KBYTES, wdst + slot * SB + (q - XLOADS) * 1024, c);
-      return;
-    }
-    if constexpr (q < XLOADS)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(in ? xrsrc : zrsrc, (lds_ptr_t)(xdst + slot * SB + q * 1024), 16,
-                                               static_cast<int>(in ? xoff[q] : zoff), kbyte, 0, 0);
-    else
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(in ? wrsrc : zrsrc, (lds_ptr_t)(wdst + slot * SB + (q - XLOADS) * 1024),
-                                               16, static_cast<int>(in ? woff[q - XLOADS] : zoff), kbyte, 0, W_AUX);
-  };
-
   typename Geom<ELT>::Acc acc[MBK][NBK];
 #pragma unroll
   for (int i = 0; i < MBK; ++i)
@@ -866,23 +844,36 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
     else xf[q - NBK][s] = *reinterpret_cast<const i32x4 *>(xfrag[hi][s] + lo + (q - NBK) * BLK * KBYTES);
   };
 
-  auto read_dyn = [&](int slot, auto R, i32x4 (&xf)[MBK][NCH], i32x4 (&wf)[NBK][NCH]) {
-    constexpr int r = decltype(R)::value;
-    constexpr int s = r / (MBK + NBK), q = r % (MBK + NBK);
-    if constexpr (q < NBK) wf[q][s] = *reinterpret_cast<const i32x4 *>(wfrag[0][s] + slot * SB + q * BLK * KBYTES);
-    else xf[q - NBK][s] = *reinterpret_cast<const i32x4 *>(xfrag[0][s] + slot * SB + (q - NBK) * BLK * KBYTES);
-  };
-
   // One k-step, number U within a run of ten (ring of five slots x two fragment sets: after ten steps
   // every slot index and register role repeats, so all of them are compile-time constants here).
   // MFMAs run on `cur` (read during the previous step), the fragments of the next step go into `nxt`,
   // and half of the fills of the pair of steps (E+4, E+5), E = U rounded down to even, are issued:
   // that pair is requested over the two steps E and E+1, row group by row group, both k-steps of a row
   // group back to back (the second one hits the line the first one brought into L1).
-  auto step = [&](auto U, int kbase, i32x4 (&xc)[MBK][NCH], i32x4 (&wc)[NBK][NCH], i32x4 (&xn)[MBK][NCH], i32x4 (&wn_)[NBK][NCH]) {
+  // GUARDED (the last steps of a tile; they start at a multiple of the trip length, so ring slots and fragment sets are
+  // the trip's): a k-step the step requests may be the partial last one of a K that is not a multiple of 64 bytes, or
+  // lie past the end of K.  Its fills go through flat addresses, per lane either its 16 bytes of the operand or, where
+  // those lie past the end of the row, 16 bytes of a page of zeros: one vector-memory instruction per fill either
+  // way, so the fill counts of the waits hold.  kb0 is the byte offset along K of step 0 of the trip, xbase / wbase
+  // (guarded steps only) the operands' first bytes.
+  auto step = [&](auto GUARDED, auto U, int64_t kb0, const uint8_t *xbase, const uint8_t *wbase, i32x4 (&xc)[MBK][NCH],
+                  i32x4 (&wc)[NBK][NCH], i32x4 (&xn)[MBK][NCH], i32x4 (&wn_)[NBK][NCH]) {
+    constexpr bool guarded = decltype(GUARDED)::value;
     constexpr int u = decltype(U)::value;
     constexpr bool even = (u & 1) == 0;
     constexpr int e0 = u & ~1;
+    const int kbase = static_cast<int>(kb0);
+    int valid[2] = {KBYTES, KBYTES};          // guarded: bytes of the two requested k-steps that lie inside K
+    int64_t gk[2] = {0, 0};                   // ... and their byte offsets along K
+    if constexpr (guarded) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int64_t kb = kb0 + (e0 + LA + h) * KBYTES;
+        const int64_t rem = c.kbytes - kb;
+        valid[h] = rem >= KBYTES ? KBYTES : (rem <= 0 ? 0 : static_cast<int>(rem));
+        gk[h] = rem > 0 ? kb : 0;
+      }
+    }
     // Stage u+1 has landed once the pair it belongs to is complete; fills are counted in issue order.
     if constexpr (even) {
       FLUXMI_WAITCNT(WAIT_EVEN, 15);  // all but the pairs requested since the one stage u+1 is in
@@ -903,7 +894,17 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
         constexpr int d = decltype(D)::value;
         constexpr int at = (d * (2 * NM) / (2 * LOADS) + 1) % (2 * NM);
         if constexpr (at == t + (even ? 0 : NM)) {
-          if constexpr (SPLIT_M0 && at % NM != 0)  // the slot before is in the same step: M0 was written there
+          if constexpr (guarded) {
+            constexpr int q = d >> 1, h = d & 1, slot = (e0 + LA + h) % STG;
+            const bool ok = c.fill_chunk * 16 < valid[h];
+            if constexpr (q < XLOADS) {
+              const uint8_t *src = ok ? xbase + gk[h] + xoff[q] : g_zero_page + lane * 16;
+              __builtin_amdgcn_global_load_lds((gbl_ptr_t)src, (lds_ptr_t)(xdst + slot * SB + q * 1024), 16, 0, 0);
+            } else {
+              const uint8_t *src = ok ? wbase + gk[h] + woff[q - XLOADS] : g_zero_page + lane * 16;
+              __builtin_amdgcn_global_load_lds((gbl_ptr_t)src, (lds_ptr_t)(wdst + slot * SB + (q - XLOADS) * 1024), 16, 0, W_AUX);
+            }
+          } else if constexpr (SPLIT_M0 && at % NM != 0)  // the slot before is in the same step: M0 was written there
             fill_go(std::integral_constant<int, (d >> 1)>{}, kbase + (e0 + LA + (d & 1)) * KBYTES);
           else
             fill_one(std::integral_constant<int, (e0 + LA + (d & 1)) % STG>{}, std::integral_constant<int, (d >> 1)>{},
@@ -913,7 +914,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
       static_for<0, 2 * LOADS>([&](auto D) {
         constexpr int d = decltype(D)::value;
         constexpr int at = (d * (2 * NM) / (2 * LOADS) + 1) % (2 * NM);
-        if constexpr (SPLIT_M0 && at % NM != 0 && at - 1 == t + (even ? 0 : NM))
+        if constexpr (!guarded && SPLIT_M0 && at % NM != 0 && at - 1 == t + (even ? 0 : NM))
           fill_m0(std::integral_constant<int, (e0 + LA + (d & 1)) % STG>{}, std::integral_constant<int, (d >> 1)>{});
       });
       mfma_slot<ELT, MBK, NBK>(t, xc, wc, acc);
@@ -922,40 +923,6 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
     FLUXMI_WAITCNT(63, 0);  // the fragments of the next step are in registers (requested long ago)
     __builtin_amdgcn_sched_barrier(0);
   };
-  // The same step with run-time ring slots (k-step ks, slot ks % 5), for the last steps of a tile, whose
-  // number is not a multiple of ten.
-  auto step_dyn = [&](int ks, bool even, i32x4 (&xc)[MBK][NCH], i32x4 (&wc)[NBK][NCH], i32x4 (&xn)[MBK][NCH], i32x4 (&wn_)[NBK][NCH]) {
-    if (even) {
-      FLUXMI_WAITCNT(WAIT_EVEN, 15);
-    } else {
-      FLUXMI_WAITCNT(WAIT_ODD, 15);
-    }
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_sched_barrier(0);
-    const int e0 = even ? ks : ks - 1;
-    const int rslot = (ks + 1) % STG, pslot0 = (e0 + LA) % STG, pslot1 = (e0 + LA + 1) % STG;
-    static_for<0, NM>([&](auto T) {
-      constexpr int t = decltype(T)::value;
-      static_for<0, NR>([&](auto R) {
-        constexpr int r = decltype(R)::value;
-        if constexpr (r * RSPAN / NR == t) read_dyn(rslot, R, xn, wn_);
-      });
-      static_for<0, 2 * LOADS>([&](auto D) {
-        constexpr int d = decltype(D)::value;
-        constexpr int at = (d * (2 * NM) / (2 * LOADS) + 1) % (2 * NM);
-        if constexpr (at < NM) {
-          if (at == t && even) fill_dyn((d & 1) ? pslot1 : pslot0, std::integral_constant<int, (d >> 1)>{}, e0 + LA + (d & 1));
-        } else {
-          if (at - NM == t && !even) fill_dyn((d & 1) ? pslot1 : pslot0, std::integral_constant<int, (d >> 1)>{}, e0 + LA + (d & 1));
-        }
-      });
-      mfma_slot<ELT, MBK, NBK>(t, xc, wc, acc);
-      __builtin_amdgcn_sched_barrier(0);
-    });
-    FLUXMI_WAITCNT(63, 0);
-    __builtin_amdgcn_sched_barrier(0);
-  };
-
   // ---- prologue: k-steps 0..3 requested as two pairs, here or by the previous tile ahead of its epilogue --
   FLUXMI_WAITCNT(0, 0);  // stores of the previous tile's epilogue (and, if it requested them, the first fills)
   if (!prefetched) issue_first_pairs<XLOADS, WLOADS>(op, smem, c);
@@ -966,22 +933,36 @@ __device__ __forceinline__ void gemm_tile(const GemmParams &p, uint8_t *smem, co
 
   // ---- main loop ----------------------------------------------------------------------------------
   // Whole trips of TRIP k-steps while every k-step a trip requests (up to TRIP - 1 + LA past its first one) is a
-  // whole one, then the remaining steps pair by pair with run-time ring slots.  An odd number of k-steps
-  // ends with a phantom step on zero fragments.
+  // whole one, then the remaining steps pair by pair with guarded fills.  An odd number of k-steps ends with a
+  // phantom step on zero fragments.
   constexpr int TRIP = Ring<MB, NB>::TRIP;
+  const int nkf = c.nkf;
   const int nfast = nkf >= TRIP + LA ? (nkf - (TRIP + LA)) / TRIP + 1 : 0;  // trips with TRIP * trip + TRIP - 1 + LA < nkf
   int kbase = 0;  // byte offset along K of step 0 of the current trip
   for (int trip = 0; trip < nfast; ++trip) {
     static_for<0, TRIP / 2>([&](auto H) {
       constexpr int u = 2 * decltype(H)::value;
-      step(std::integral_constant<int, u>{}, kbase, xa, wa, xb, wb);
-      step(std::integral_constant<int, u + 1>{}, kbase, xb, wb, xa, wa);
+      step(std::false_type{}, std::integral_constant<int, u>{}, kbase, nullptr, nullptr, xa, wa, xb, wb);
+      step(std::false_type{}, std::integral_constant<int, u + 1>{}, kbase, nullptr, nullptr, xb, wb, xa, wa);
     });
     kbase += TRIP * KBYTES;
   }
-  for (int ks = TRIP * nfast; ks < nk; ks += 2) {
-    step_dyn(ks, true, xa, wa, xb, wb);
-    step_dyn(ks + 1, false, xb, wb, xa, wa);
+  if (TRIP * nfast < nk) {
+    const KernArgs pe = kernel_args();
+    const uint8_t *xbase = pe->gather_a != nullptr ? pe->a : pe->a + static_cast<int64_t>(row_base + m0) * c.kbytes;
+    int n0g = t.n0;
+    const int gg = split_group(n0g, pe->n, pe->ngroups);
+    const uint8_t *wbase = pe->b[gg] + (static_cast<int64_t>(e) * pe->n + n0g) * c.kbytes;
+    int64_t kb = static_cast<int64_t>(kbase);
+    for (int ks = TRIP * nfast; ks < nk; ks += TRIP, kb += TRIP * KBYTES) {
+      static_for<0, TRIP / 2>([&](auto H) {
+        constexpr int u = 2 * decltype(H)::value;
+        if (ks + u < nk) {
+          step(std::true_type{}, std::integral_constant<int, u>{}, kb, xbase, wbase, xa, wa, xb, wb);
+          step(std::true_type{}, std::integral_constant<int, u + 1>{}, kb, xbase, wbase, xb, wb, xa, wa);
+        }
+      });
+    }
   }
 
   // ---- epilogue ---------------------------------------------------------------------------------
