@@ -32,7 +32,7 @@ PEAK_SCLK_MHZ = 2400.0
 # HBM bytes per grouped-GEMM launch on C3 (mean of layer0 and layer1): FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000
 # from the two rocprofv3 --pmc runs summarised in profiles/bench_c3_pmc_counters.md (scale factors from the
 # 1 GiB copy of --calib-copy).  Only valid for the C3 workload with the fp32 layer1 intermediate.
-GEMM_TRAFFIC_C3_BYTES = 4.56e9
+GEMM_TRAFFIC_C3_BYTES = 4.47e9
 
 
 def parse():
