@@ -14,7 +14,7 @@ void set_error(const char *fmt, ...) {
 }
 }  // namespace fluxmi
 
-extern "C" int fluxmi_version(void) { return 110; }
+extern "C" int fluxmi_version(void) { return 111; }
 
 extern "C" const char *fluxmi_last_error(void) { return fluxmi::g_last_error; }
 
